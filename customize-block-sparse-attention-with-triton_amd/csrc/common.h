@@ -1,0 +1,44 @@
+// Shared declarations of the library's translation units (not part of the public ABI).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "bsattn.h"
+
+#define BSATTN_VERSION 100
+
+namespace bsattn {
+
+// mask_index.hip
+int launch_reduce_dense_mask(const uint8_t* dense, int Bm, int Hm, int N, int64_t sb, int64_t sh,
+                             int64_t sm, uint8_t* block_out, hipStream_t st);
+int launch_block_mask_to_lists(const uint8_t* block, int Bm, int Hm, int nb, int64_t sb, int64_t sh,
+                               int64_t sm, int64_t sn, int32_t* row_ptr, int32_t* col_idx,
+                               int32_t* groups, int32_t* counts, int32_t* ws, hipStream_t st);
+
+struct AttnShape {
+  int B, H, N, D, Bm, Hm;
+  int dtype, out_dtype;
+  float sm_scale;
+  int64_t qs[3], ks[3], vs[3], os[3], dos[3];  // batch, head, row strides (elements)
+};
+
+// attn_fwd.hip
+size_t fwd_workspace_bytes(int B, int H, int N, int D);
+int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
+               const int32_t* row_ptr, const int32_t* col_idx, const AttnShape& s, void* ws,
+               hipStream_t st);
+
+// attn_bwd.hip
+size_t bwd_workspace_bytes(int B, int H, int N, int D);
+int launch_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
+               const float* lse, void* dq, void* dk, void* dv, const int32_t* row_ptr,
+               const int32_t* col_idx, const int32_t* col_ptr, const int32_t* row_idx,
+               const AttnShape& s, void* ws, hipStream_t st);
+
+// reorder.hip
+int launch_reorder(const void* x, void* out, int BS, int NH, int F, int Hh, int W, int row_bytes,
+                   const int32_t* orders, const int32_t* inv_orders, hipStream_t st);
+
+inline int launch_status() { return hipGetLastError() == hipSuccess ? BSATTN_OK : BSATTN_ERR_LAUNCH; }
+
+}  // namespace bsattn

@@ -1,0 +1,139 @@
+// Mask preprocessing: elementwise mask -> block mask -> kept-tile lists.
+// Integer/byte work bound by HBM bandwidth; output is bit-identical to the reference's
+// build_groups_from_block_mask (fa2_custom_mask/fa2_custom_mask.py:15-38).
+#include "common.h"
+
+namespace bsattn {
+
+// ---------------------------------------------------------------------------------------
+// dense [.,.,N,N] bool -> block [.,.,nb,nb] bool (tile kept iff any element set).
+// One wavefront owns 64 rows x 1024 columns (16 tiles): every lane ORs its 16-byte column
+// slice over the 64 rows, then a ballot folds 4 lanes into one tile flag.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void reduce_dense_kernel(const uint8_t* __restrict__ dense, int N,
+                                                           int nb, int H, int64_t sb, int64_t sh,
+                                                           int64_t sm, uint8_t* __restrict__ block) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int rb = blockIdx.x;
+  const int col0 = (blockIdx.y * 4 + wave) * 1024;
+  if (col0 >= N) return;
+  const int bh = blockIdx.z;
+  const int b = bh / H, h = bh % H;
+  const int col = col0 + lane * 16;
+  const bool in = col < N;
+  const uint8_t* p = dense + b * sb + h * sh + (int64_t)rb * 64 * sm + (in ? col : 0);
+  typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
+  uintx4 acc = {0u, 0u, 0u, 0u};
+#pragma unroll 16
+  for (int r = 0; r < 64; ++r) acc |= __builtin_nontemporal_load(reinterpret_cast<const uintx4*>(p + r * sm));
+  const bool nz = in && ((acc[0] | acc[1] | acc[2] | acc[3]) != 0u);
+  const unsigned long long bal = __ballot(nz);
+  if (lane < 16) {
+    const int t = (col0 >> 6) + lane;
+    if (t < nb) block[((int64_t)bh * nb + rb) * nb + t] = ((bal >> (4 * lane)) & 0xFull) ? 1 : 0;
+  }
+}
+
+// one wavefront per mask row: number of kept tiles
+__global__ __launch_bounds__(256) void count_rows_kernel(const uint8_t* __restrict__ block, int rows,
+                                                         int nb, int H, int64_t sb, int64_t sh,
+                                                         int64_t sm, int64_t sn,
+                                                         int32_t* __restrict__ cnt) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int m = row % nb, bh = row / nb;
+  const uint8_t* p = block + (bh / H) * sb + (bh % H) * sh + (int64_t)m * sm;
+  int c = 0;
+  for (int n0 = 0; n0 < nb; n0 += 64) {
+    const int n = n0 + lane;
+    const bool keep = n < nb && p[(int64_t)n * sn] != 0;
+    c += __popcll(__ballot(keep));
+  }
+  if (lane == 0) cnt[row] = c;
+}
+
+// single workgroup: exclusive scan of the per-row counts (row_ptr) and of the non-empty
+// flags (position of each row in `groups`); totals to counts[0..1].
+__global__ __launch_bounds__(1024) void scan_rows_kernel(const int32_t* __restrict__ cnt, int rows,
+                                                         int32_t* __restrict__ row_ptr,
+                                                         int32_t* __restrict__ gidx,
+                                                         int32_t* __restrict__ counts) {
+  __shared__ int s_t[1024];
+  __shared__ int s_g[1024];
+  const int tid = threadIdx.x;
+  const int per = (rows + 1023) / 1024;
+  const int r0 = min(rows, tid * per), r1 = min(rows, r0 + per);
+  int t = 0, g = 0;
+  for (int r = r0; r < r1; ++r) { const int c = cnt[r]; t += c; g += c > 0; }
+  s_t[tid] = t; s_g[tid] = g;
+  __syncthreads();
+  for (int off = 1; off < 1024; off <<= 1) {   // Hillis-Steele inclusive scan
+    int at = 0, ag = 0;
+    if (tid >= off) { at = s_t[tid - off]; ag = s_g[tid - off]; }
+    __syncthreads();
+    s_t[tid] += at; s_g[tid] += ag;
+    __syncthreads();
+  }
+  int bt = s_t[tid] - t, bg = s_g[tid] - g;    // exclusive prefix of this thread's span
+  for (int r = r0; r < r1; ++r) {
+    const int c = cnt[r];
+    row_ptr[r] = bt; gidx[r] = bg;
+    bt += c; bg += c > 0;
+  }
+  if (tid == 1023) { row_ptr[rows] = s_t[1023]; counts[0] = s_g[1023]; counts[1] = s_t[1023]; }
+}
+
+// one wavefront per mask row: ordered fill of col_idx and the row's `groups` entry
+__global__ __launch_bounds__(256) void fill_rows_kernel(const uint8_t* __restrict__ block, int rows,
+                                                        int nb, int H, int64_t sb, int64_t sh,
+                                                        int64_t sm, int64_t sn,
+                                                        const int32_t* __restrict__ row_ptr,
+                                                        const int32_t* __restrict__ gidx,
+                                                        int32_t* __restrict__ col_idx,
+                                                        int32_t* __restrict__ groups) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int m = row % nb, bh = row / nb;
+  const uint8_t* p = block + (bh / H) * sb + (bh % H) * sh + (int64_t)m * sm;
+  const int start = row_ptr[row];
+  int pos = start;
+  for (int n0 = 0; n0 < nb; n0 += 64) {
+    const int n = n0 + lane;
+    const bool keep = n < nb && p[(int64_t)n * sn] != 0;
+    const unsigned long long bal = __ballot(keep);
+    if (keep) col_idx[pos + __popcll(bal & ((1ull << lane) - 1ull))] = n;
+    pos += __popcll(bal);
+  }
+  if (groups != nullptr && lane == 0 && pos > start) {
+    int32_t* g = groups + (int64_t)gidx[row] * 5;
+    g[0] = bh / H; g[1] = bh % H; g[2] = m; g[3] = start; g[4] = pos - start;
+  }
+}
+
+int launch_reduce_dense_mask(const uint8_t* dense, int Bm, int Hm, int N, int64_t sb, int64_t sh,
+                             int64_t sm, uint8_t* block_out, hipStream_t st) {
+  const int nb = N / 64;
+  dim3 grid(nb, (N + 4095) / 4096, Bm * Hm);
+  hipLaunchKernelGGL(reduce_dense_kernel, grid, dim3(256), 0, st, dense, N, nb, Hm, sb, sh, sm,
+                     block_out);
+  return launch_status();
+}
+
+int launch_block_mask_to_lists(const uint8_t* block, int Bm, int Hm, int nb, int64_t sb, int64_t sh,
+                               int64_t sm, int64_t sn, int32_t* row_ptr, int32_t* col_idx,
+                               int32_t* groups, int32_t* counts, int32_t* ws, hipStream_t st) {
+  const int rows = Bm * Hm * nb;
+  int32_t* cnt = ws;
+  int32_t* gidx = ws + rows;
+  const dim3 grid((rows + 3) / 4);
+  hipLaunchKernelGGL(count_rows_kernel, grid, dim3(256), 0, st, block, rows, nb, Hm, sb, sh, sm, sn,
+                     cnt);
+  hipLaunchKernelGGL(scan_rows_kernel, dim3(1), dim3(1024), 0, st, cnt, rows, row_ptr, gidx, counts);
+  hipLaunchKernelGGL(fill_rows_kernel, grid, dim3(256), 0, st, block, rows, nb, Hm, sb, sh, sm, sn,
+                     row_ptr, gidx, col_idx, groups);
+  return launch_status();
+}
+
+}  // namespace bsattn

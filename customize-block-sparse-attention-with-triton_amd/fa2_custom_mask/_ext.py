@@ -1,0 +1,87 @@
+"""ctypes binding of libbsattn.so, the C-ABI library holding the gfx950 kernels.
+
+There is deliberately no fallback: if the library is missing, or a call returns an error
+code, a RuntimeError is raised.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.environ.get("BSATTN_LIB", os.path.join(_HERE, "libbsattn.so"))
+_lib = None
+
+F16, BF16, F32 = 0, 1, 2
+_DTYPE_CODE = {torch.float16: F16, torch.bfloat16: BF16, torch.float32: F32}
+
+_i, _i64, _p, _f = ctypes.c_int, ctypes.c_int64, ctypes.c_void_p, ctypes.c_float
+_SIGNATURES = {
+    "bsattn_version": ([], _i),
+    "bsattn_strerror": ([_i], ctypes.c_char_p),
+    "bsattn_reduce_dense_mask": ([_p, _i, _i, _i, _i64, _i64, _i64, _p, _p], _i),
+    "bsattn_mask_lists_workspace": ([_i, _i, _i, ctypes.POINTER(ctypes.c_size_t)], _i),
+    "bsattn_block_mask_to_lists": ([_p, _i, _i, _i, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p,
+                                    ctypes.c_size_t, _p], _i),
+    "bsattn_fwd_workspace": ([_i, _i, _i, _i, ctypes.POINTER(ctypes.c_size_t)], _i),
+    "bsattn_fwd": ([_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f,
+                    _p, _p, _p, _p, _p, ctypes.c_size_t, _p], _i),
+    "bsattn_bwd_workspace": ([_i, _i, _i, _i, ctypes.POINTER(ctypes.c_size_t)], _i),
+    "bsattn_bwd": ([_p] * 13 + [_i] * 8 + [_f] + [_p] * 5 + [_p, ctypes.c_size_t, _p], _i),
+    "bsattn_reorder": ([_p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p], _i),
+}
+EXPORTS = tuple(_SIGNATURES)
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "libbsattn.so not found at %s: build it with "
+                "`python customize-block-sparse-attention-with-triton_amd/build.py`" % LIB_PATH)
+        l = ctypes.CDLL(LIB_PATH)
+        for name, (argtypes, restype) in _SIGNATURES.items():
+            fn = getattr(l, name)
+            fn.argtypes = argtypes
+            fn.restype = restype
+        _lib = l
+    return _lib
+
+
+def check(rc, what):
+    if rc != 0:
+        raise RuntimeError("%s failed: %s (code %d)" % (what, lib().bsattn_strerror(rc).decode(), rc))
+
+
+def dtype_code(dt):
+    try:
+        return _DTYPE_CODE[dt]
+    except KeyError:
+        raise TypeError("unsupported dtype %s" % dt)
+
+
+def strides4(t):
+    return (ctypes.c_int64 * 4)(*t.stride())
+
+
+def current_stream(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def mask_lists_workspace(Bm, Hm, nb):
+    n = ctypes.c_size_t()
+    check(lib().bsattn_mask_lists_workspace(Bm, Hm, nb, ctypes.byref(n)), "bsattn_mask_lists_workspace")
+    return n.value
+
+
+def fwd_workspace(B, H, N, D):
+    n = ctypes.c_size_t()
+    check(lib().bsattn_fwd_workspace(B, H, N, D, ctypes.byref(n)), "bsattn_fwd_workspace")
+    return n.value
+
+
+def bwd_workspace(B, H, N, D):
+    n = ctypes.c_size_t()
+    check(lib().bsattn_bwd_workspace(B, H, N, D, ctypes.byref(n)), "bsattn_bwd_workspace")
+    return n.value

@@ -1,0 +1,151 @@
+"""Host boundary of the block-sparse attention operator.
+
+Mirrors fa2_custom_mask/fa2_custom_mask.py of the reference: `build_groups_from_block_mask`
+(:15-38) and the autograd function behind `flash_attention_custom_mask` (:40-157), with the
+device work done by hand-written gfx950 kernels reached through the C ABI in include/bsattn.h.
+"""
+import ctypes
+
+import torch
+
+from . import _ext
+from .utils import TILE, block_mask_to_lists, to_block_mask, _check_mask
+
+
+def build_groups_from_block_mask(mask):
+    """Same contract as the reference (fa2_custom_mask.py:15-38): bool [B,H,nb,nb] ->
+    (groups int32 [G,5] = (b,h,m_block,start,length), n_list int32 [T]) on mask.device, rows
+    without a kept tile omitted, (None, None) if nothing is kept.  The lists are produced by
+    the GPU kernels; only the two sizes G and T are read back to shape the result."""
+    assert mask.dtype == torch.bool                                   # :20
+    _check_mask(mask)
+    lists = block_mask_to_lists(mask, want_groups=True)
+    G, T = lists.counts.tolist()
+    if G == 0:                                                        # :34-35
+        return None, None
+    return lists.groups[:G].contiguous(), lists.col_idx[:T].contiguous()   # :36-38
+
+
+def _prep(x):
+    """Kernels need unit stride along the head dimension and 16-byte aligned rows."""
+    if x.stride(3) != 1 or any((s * x.element_size()) % 16 for s in x.stride()[:3]) or x.data_ptr() % 16:
+        return x.contiguous()
+    return x
+
+
+def _check_qkv(q, k, v, mask):
+    if not (q.is_cuda and k.is_cuda and v.is_cuda):
+        raise RuntimeError("q, k, v must be GPU tensors (there is no CPU path)")
+    if q.dim() != 4 or k.shape != q.shape or v.shape != q.shape:
+        raise ValueError("q, k, v must share one shape [B, H, N, D]")   # :53-57
+    if q.dtype not in (torch.float16, torch.bfloat16) or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise TypeError("q, k, v must all be float16 or all bfloat16")
+    B, H, N, D = q.shape
+    if D not in (64, 128):                                             # :58 and fa2_fwd.py:120
+        raise ValueError("head dimension must be 64 or 128")
+    if N % TILE != 0:
+        raise ValueError("sequence length must be a multiple of 64")
+    if mask is None:
+        raise ValueError("mask=None is not supported (the reference has no dense path either: "
+                         "`groups` is unbound at fa2_custom_mask.py:69)")
+    _check_mask(mask)
+    if mask.shape[0] not in (1, B) or mask.shape[1] not in (1, H):
+        raise ValueError("mask batch/head sizes must be 1 or match q")
+    return B, H, N, D
+
+
+def _forward(q, k, v, lists, sm_scale, out_dtype, want_lse):
+    B, H, N, D = q.shape
+    q, k, v = _prep(q), _prep(k), _prep(v)
+    o = torch.empty((B, H, N, D), dtype=out_dtype, device=q.device)            # :59
+    lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device) if want_lse else None  # :70
+    wsb = _ext.fwd_workspace(B, H, N, D)
+    ws = torch.empty(wsb, dtype=torch.uint8, device=q.device)
+    rc = _ext.lib().bsattn_fwd(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr() if want_lse else None,
+        lists.row_ptr.data_ptr(), lists.col_idx.data_ptr(), lists.Bm, lists.Hm, B, H, N, D,
+        _ext.dtype_code(q.dtype), _ext.dtype_code(out_dtype), float(sm_scale),
+        _ext.strides4(q), _ext.strides4(k), _ext.strides4(v), _ext.strides4(o),
+        ws.data_ptr(), wsb, _ext.current_stream(q.device))
+    _ext.check(rc, "bsattn_fwd")
+    return o, lse
+
+
+def _backward(q, k, v, o, do, lse, lists, lists_t, sm_scale, out_dtype):
+    B, H, N, D = q.shape
+    q, k, v, o, do = _prep(q), _prep(k), _prep(v), _prep(o), _prep(do)
+    dq = torch.empty((B, H, N, D), dtype=out_dtype, device=q.device)           # :101-103
+    dk = torch.empty_like(dq)
+    dv = torch.empty_like(dq)
+    wsb = _ext.bwd_workspace(B, H, N, D)
+    ws = torch.empty(wsb, dtype=torch.uint8, device=q.device)
+    rc = _ext.lib().bsattn_bwd(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(), lse.data_ptr(),
+        dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+        lists.row_ptr.data_ptr(), lists.col_idx.data_ptr(), lists_t.row_ptr.data_ptr(),
+        lists_t.col_idx.data_ptr(), lists.Bm, lists.Hm, B, H, N, D,
+        _ext.dtype_code(q.dtype), _ext.dtype_code(out_dtype), float(sm_scale),
+        _ext.strides4(q), _ext.strides4(k), _ext.strides4(v), _ext.strides4(o), _ext.strides4(do),
+        ws.data_ptr(), wsb, _ext.current_stream(q.device))
+    _ext.check(rc, "bsattn_bwd")
+    return dq, dk, dv
+
+
+class _attention(torch.autograd.Function):
+    """forward(q, k, v, mask, sm_scale) as the reference (fa2_custom_mask.py:43-94); two extra
+    trailing arguments select an fp32 output and the LSE as second result."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, mask=None, sm_scale=1.3, out_fp32=False, return_lse=False):
+        B, H, N, D = _check_qkv(q, k, v, mask)
+        block = to_block_mask(mask, N)
+        lists = block_mask_to_lists(block)                                   # :48
+        out_dtype = torch.float32 if out_fp32 else q.dtype
+        o, lse = _forward(q, k, v, lists, sm_scale, out_dtype, True)
+        ctx.save_for_backward(q, k, v, o, lse, block)                        # :89
+        ctx.lists = lists
+        ctx.sm_scale = sm_scale
+        ctx.out_dtype = out_dtype
+        ctx.return_lse = return_lse
+        if return_lse:
+            ctx.mark_non_differentiable(lse)
+            return o, lse
+        return o                                                              # :94
+
+    @staticmethod
+    def backward(ctx, do, *unused):
+        q, k, v, o, lse, block = ctx.saved_tensors
+        lists_t = block_mask_to_lists(block, transpose=True)
+        o_in = o if o.dtype == q.dtype else o.to(q.dtype)
+        do_in = do if do.dtype == q.dtype else do.to(q.dtype)
+        # autograd hands gradients back in the dtype of q, k, v
+        dq, dk, dv = _backward(q, k, v, o_in, do_in, lse, ctx.lists, lists_t, ctx.sm_scale, q.dtype)
+        return dq, dk, dv, None, None, None, None                            # :155
+
+
+def flash_attention_custom_mask(q, k, v, mask=None, sm_scale=1.3):
+    """Drop-in for the reference's `flash_attention_custom_mask = _attention.apply`
+    (fa2_custom_mask.py:157): q,k,v [B,H,N,D] fp16/bf16 on the GPU, mask bool
+    [B|1,H|1,N/64,N/64] (or elementwise [B|1,H|1,N,N]), returns o like q."""
+    return _attention.apply(q, k, v, mask, sm_scale)
+
+
+def flash_attention_custom_mask_lse(q, k, v, mask, sm_scale, out_fp32=False):
+    """Same operator, also returning the natural-log logsumexp [B,H,N] fp32 of the kept scaled
+    scores; out_fp32=True returns O in fp32.  (Not in the reference, whose second output M is
+    only the running maximum: fa2_fwd.py:194-196.)"""
+    return _attention.apply(q, k, v, mask, sm_scale, out_fp32, True)
+
+
+def attention_forward_backward(q, k, v, mask, sm_scale, do, out_fp32=False):
+    """Non-autograd entry: (o, lse, dq, dk, dv) in one call; with out_fp32 all five results
+    are fp32 (autograd itself can only hand back gradients in the dtype of q)."""
+    B, H, N, D = _check_qkv(q, k, v, mask)
+    block = to_block_mask(mask, N)
+    lists = block_mask_to_lists(block)
+    lists_t = block_mask_to_lists(block, transpose=True)
+    out_dtype = torch.float32 if out_fp32 else q.dtype
+    o, lse = _forward(q, k, v, lists, sm_scale, out_dtype, True)
+    o_in = o if o.dtype == q.dtype else o.to(q.dtype)
+    dq, dk, dv = _backward(q, k, v, o_in, do.to(q.dtype), lse, lists, lists_t, sm_scale, out_dtype)
+    return o, lse, dq, dk, dv

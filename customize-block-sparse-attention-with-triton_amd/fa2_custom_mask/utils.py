@@ -1,0 +1,100 @@
+"""Mask preprocessing on the GPU and small helpers.
+
+`is_hip` / `keep` keep the names exported by the reference (fa2_custom_mask/utils.py:3-14).
+"""
+import ctypes
+
+import torch
+
+from . import _ext
+
+TILE = 64
+
+
+def is_hip():
+    """The reference hard-wires False (fa2_custom_mask/utils.py:3-4); this build only runs on HIP."""
+    return True
+
+
+def keep(conf):
+    """Autotune filter of the reference (fa2_custom_mask/utils.py:9-14).  There is no autotuner
+    here; every configuration is kept."""
+    return True
+
+
+class TileLists:
+    """Device-resident kept-tile lists of a block mask [Bm, Hm, nb, nb] (fixed shapes, no
+    host synchronisation): row_ptr int32 [Bm*Hm*nb+1], col_idx int32 [Bm*Hm*nb*nb] (first T
+    entries valid), counts int32 [2] = (G, T), groups int32 [Bm*Hm*nb, 5] (first G rows
+    valid) or None."""
+
+    __slots__ = ("row_ptr", "col_idx", "groups", "counts", "Bm", "Hm", "nb")
+
+    def __init__(self, row_ptr, col_idx, groups, counts, Bm, Hm, nb):
+        self.row_ptr, self.col_idx, self.groups, self.counts = row_ptr, col_idx, groups, counts
+        self.Bm, self.Hm, self.nb = Bm, Hm, nb
+
+
+def _check_mask(mask):
+    if not isinstance(mask, torch.Tensor) or mask.dtype != torch.bool:
+        raise TypeError("mask must be a torch.bool tensor")       # fa2_custom_mask.py:20
+    if mask.dim() != 4:
+        raise ValueError("mask must have 4 dimensions [B, H, rows, cols]")
+    if not mask.is_cuda:
+        raise RuntimeError("mask must live on the GPU")
+
+
+def reduce_dense_mask(mask):
+    """Elementwise mask [Bm,Hm,N,N] -> block mask [Bm,Hm,N/64,N/64] (tile kept iff any element
+    set; exact inverse of the expansion at kernel-test.py:18 for tile-constant masks)."""
+    _check_mask(mask)
+    Bm, Hm, N, N2 = mask.shape
+    if N != N2 or N % TILE != 0:
+        raise ValueError("dense mask must be [.., N, N] with N a multiple of 64")
+    if mask.stride(3) != 1 or any(s % 16 for s in mask.stride()[:3]) or mask.data_ptr() % 16:
+        mask = mask.contiguous()
+    nb = N // TILE
+    block = torch.empty((Bm, Hm, nb, nb), dtype=torch.bool, device=mask.device)
+    rc = _ext.lib().bsattn_reduce_dense_mask(mask.data_ptr(), Bm, Hm, N, mask.stride(0), mask.stride(1),
+                                             mask.stride(2), block.data_ptr(),
+                                             _ext.current_stream(mask.device))
+    _ext.check(rc, "bsattn_reduce_dense_mask")
+    return block
+
+
+def block_mask_to_lists(block, transpose=False, want_groups=False):
+    """Block mask -> TileLists.  transpose=True lists, for every column block, the kept row
+    blocks (what the dK/dV pass walks)."""
+    _check_mask(block)
+    Bm, Hm, nb, nb2 = block.shape
+    if nb != nb2:
+        raise ValueError("block mask must be square")
+    dev = block.device
+    rows = Bm * Hm * nb
+    row_ptr = torch.empty(rows + 1, dtype=torch.int32, device=dev)
+    col_idx = torch.empty(rows * nb, dtype=torch.int32, device=dev)
+    groups = torch.empty((rows, 5), dtype=torch.int32, device=dev) if want_groups else None
+    counts = torch.empty(2, dtype=torch.int32, device=dev)
+    wsb = _ext.mask_lists_workspace(Bm, Hm, nb)
+    ws = torch.empty(wsb, dtype=torch.uint8, device=dev)
+    sb, sh, sm, sn = block.stride()
+    if transpose:
+        sm, sn = sn, sm
+    rc = _ext.lib().bsattn_block_mask_to_lists(
+        block.data_ptr(), Bm, Hm, nb, sb, sh, sm, sn, row_ptr.data_ptr(), col_idx.data_ptr(),
+        groups.data_ptr() if want_groups else None, counts.data_ptr(), ws.data_ptr(), wsb,
+        _ext.current_stream(dev))
+    _ext.check(rc, "bsattn_block_mask_to_lists")
+    return TileLists(row_ptr, col_idx, groups, counts, Bm, Hm, nb)
+
+
+def to_block_mask(mask, N):
+    """Accepts the reference's block form [.,.,N/64,N/64] or an elementwise [.,.,N,N] mask."""
+    _check_mask(mask)
+    nb = N // TILE
+    if mask.shape[2] == nb and mask.shape[3] == nb:
+        return mask
+    if mask.shape[2] == N and mask.shape[3] == N:
+        return reduce_dense_mask(mask)
+    raise ValueError("mask shape %s matches neither [.., %d, %d] nor [.., %d, %d]"
+                     % (tuple(mask.shape), nb, nb, N, N))

@@ -1,0 +1,147 @@
+/*
+ * bsattn.h - C ABI of libbsattn.so: block-sparse FlashAttention-2 for AMD MI355X (gfx950).
+ *
+ * This is the boundary a replacement for the reference's device layer binds to.  The
+ * reference has no native FFI of its own (its device code is Triton JIT launched from
+ * Python); each entry point below names the reference Python/Triton interface it
+ * replaces, with paths relative to the reference repository root.
+ *
+ * Conventions
+ *   - plain C types only; every function returns 0 (BSATTN_OK) or a negative error code;
+ *   - all argument validation happens before any device work, so error paths can be
+ *     exercised on a host without a GPU;
+ *   - all buffers are caller-owned device memory (raw pointers, e.g. tensor.data_ptr());
+ *     the library never allocates or frees device memory: scratch is passed in as a
+ *     workspace whose size is queried first;
+ *   - every call only enqueues work on `stream` (a hipStream_t passed as void*, NULL = the
+ *     default stream) and never synchronises;
+ *   - strides are in elements, int64; tiles are fixed 64x64 (reference:
+ *     fa2_custom_mask/fa2_fwd.py:13-14).
+ */
+#ifndef BSATTN_H_
+#define BSATTN_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BSATTN_TILE 64
+
+/* error codes */
+#define BSATTN_OK 0
+#define BSATTN_ERR_NULL (-1)       /* a required pointer is NULL */
+#define BSATTN_ERR_SHAPE (-2)      /* non-positive size, N not a multiple of 64, bad broadcast */
+#define BSATTN_ERR_DTYPE (-3)      /* unknown dtype code */
+#define BSATTN_ERR_HEAD_DIM (-4)   /* head dimension not in {64, 128} */
+#define BSATTN_ERR_STRIDE (-5)     /* innermost stride != 1 or rows not 16-byte aligned */
+#define BSATTN_ERR_WORKSPACE (-6)  /* workspace NULL or too small */
+#define BSATTN_ERR_LAUNCH (-7)     /* the HIP runtime refused a launch */
+#define BSATTN_ERR_RANGE (-8)      /* a size exceeds what 32-bit indices can address */
+
+/* dtype codes */
+#define BSATTN_F16 0
+#define BSATTN_BF16 1
+#define BSATTN_F32 2 /* outputs only */
+
+int bsattn_version(void);
+/* Static string for an error code; never freed by the caller. */
+const char* bsattn_strerror(int code);
+
+/* ------------------------------------------------------------------------------------
+ * Mask preprocessing (integer work, bit-exact).
+ * Replaces build_groups_from_block_mask, fa2_custom_mask/fa2_custom_mask.py:15-38, which
+ * the reference runs as a Python triple loop with one torch.nonzero + host sync per row.
+ * ---------------------------------------------------------------------------------- */
+
+/* Reduce an elementwise mask [Bm,Hm,N,N] (bool bytes, innermost stride 1, row stride a
+ * multiple of 16 and a 16-byte aligned base) to a block mask [Bm,Hm,N/64,N/64]
+ * (contiguous bool bytes): a tile is kept iff any of its 64x64 elements is set.  This is
+ * the inverse of the expansion at kernel-test.py:18 for tile-constant masks. */
+int bsattn_reduce_dense_mask(const uint8_t* dense, int Bm, int Hm, int N,
+                             int64_t sb, int64_t sh, int64_t sm,
+                             uint8_t* block_out, void* stream);
+
+/* Bytes of workspace bsattn_block_mask_to_lists needs for Bm*Hm*nb rows. */
+int bsattn_mask_lists_workspace(int Bm, int Hm, int nb, size_t* bytes);
+
+/* Block mask [Bm,Hm,nb,nb] (bool bytes, arbitrary element strides; pass the row/column
+ * strides swapped to obtain the column lists a backward pass needs) -> kept-tile lists:
+ *   row_ptr  int32 [Bm*Hm*nb + 1]  exclusive prefix sum of kept tiles per row
+ *   col_idx  int32 [capacity Bm*Hm*nb*nb]  ascending kept column tiles, row after row
+ *                                  (identical to the reference's n_list)
+ *   groups   int32 [capacity Bm*Hm*nb, 5] or NULL: the reference's (b,h,m_block,start,len)
+ *                                  rows with empty rows omitted (fa2_custom_mask.py:29-33)
+ *   counts   int32 [2]: G (rows of `groups`) and T (kept tiles); (0,0) corresponds to the
+ *                                  reference returning (None, None) (fa2_custom_mask.py:34-35)
+ */
+int bsattn_block_mask_to_lists(const uint8_t* block, int Bm, int Hm, int nb,
+                               int64_t sb, int64_t sh, int64_t sm, int64_t sn,
+                               int32_t* row_ptr, int32_t* col_idx, int32_t* groups,
+                               int32_t* counts, void* workspace, size_t workspace_bytes,
+                               void* stream);
+
+/* ------------------------------------------------------------------------------------
+ * Forward.  Replaces the launch of _attn_fwd (fa2_custom_mask/fa2_fwd.py:108-206) from
+ * _attention.forward (fa2_custom_mask/fa2_custom_mask.py:69-87).
+ * ---------------------------------------------------------------------------------- */
+
+/* Bytes of workspace bsattn_fwd needs (partial results of row blocks whose kept-tile list
+ * is split over several wavefronts). */
+int bsattn_fwd_workspace(int B, int H, int N, int D, size_t* bytes);
+
+/* q,k,v: [B,H,N,D] fp16/bf16 (dtype), strides[4] each, innermost stride 1.
+ * o:     [B,H,N,D] of out_dtype (dtype itself or BSATTN_F32), strides o_strides.
+ * lse:   fp32 [B,H,N] contiguous or NULL: natural-log logsumexp of the kept scaled scores.
+ *        (The reference's M output, fa2_fwd.py:194-196, is the running maximum only and is
+ *        not reproduced.)
+ * row_ptr/col_idx: lists from bsattn_block_mask_to_lists for a [Bm,Hm,nb,nb] mask,
+ *        Bm in {1,B}, Hm in {1,H} (1 = shared across that axis).
+ * Row blocks without a kept tile get O = 0 and lse = -inf (the reference leaves them
+ * unwritten: fa2_custom_mask.py:29-30,59). */
+int bsattn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
+               const int32_t* row_ptr, const int32_t* col_idx, int Bm, int Hm,
+               int B, int H, int N, int D, int dtype, int out_dtype, float sm_scale,
+               const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+               const int64_t* o_strides, void* workspace, size_t workspace_bytes,
+               void* stream);
+
+/* ------------------------------------------------------------------------------------
+ * Backward.  Replaces _attn_bwd_preprocess and _attn_bwd (fa2_custom_mask/fa2_bwd.py:5-19,
+ * 140-285) as launched from _attention.backward (fa2_custom_mask/fa2_custom_mask.py:97-155).
+ * The gradient algebra is the reference's (fa2_bwd.py:17,57-74,117-130,232,284) evaluated
+ * over exactly the kept tiles.
+ * ---------------------------------------------------------------------------------- */
+int bsattn_bwd_workspace(int B, int H, int N, int D, size_t* bytes);
+
+/* q,k,v,o,d_o: [B,H,N,D] fp16/bf16 with their own strides; lse from bsattn_fwd.
+ * dq,dk,dv: [B,H,N,D] of out_dtype, contiguous.
+ * row_ptr/col_idx: row lists; col_ptr/row_idx: column lists (the same call with the mask's
+ * row and column strides swapped). */
+int bsattn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
+               const float* lse, void* dq, void* dk, void* dv,
+               const int32_t* row_ptr, const int32_t* col_idx,
+               const int32_t* col_ptr, const int32_t* row_idx, int Bm, int Hm,
+               int B, int H, int N, int D, int dtype, int out_dtype, float sm_scale,
+               const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+               const int64_t* o_strides, const int64_t* do_strides,
+               void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------
+ * Head-wise token reorder.  Replaces reorder_kernel / inv_reorder_kernel
+ * (fa2_custom_mask/permute.py:5-58, 60-126) as launched from apply_head_wise_reorder /
+ * apply_inv_reorder (fa2_custom_mask/functional.py:5-20, 46-62).
+ * x,out: [BS,NH,F*Hh*W,D] contiguous, elem_bytes per element (row bytes a multiple of 4);
+ * orders: int32 [NH,3] device memory; inv_orders: int32 [NH,3] or NULL (forward reorder).
+ * out[b,h,new_t,:] = x[b,h,t,:] with new_t as permute.py:45-52.
+ * ---------------------------------------------------------------------------------- */
+int bsattn_reorder(const void* x, void* out, int BS, int NH, int F, int Hh, int W, int D,
+                   int elem_bytes, const int32_t* orders, const int32_t* inv_orders,
+                   void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BSATTN_H_ */

@@ -1,0 +1,126 @@
+"""GPU parity of the forward kernel against the CPU oracle's naive fp32 masked softmax
+(kernel-test.py:37-40).  Tolerances: max-abs 2e-2 (fp16) / 3e-2 (bf16), rel-L2 1e-3 (for bf16
+the rel-L2 bar applies to the fp32-output mode: rounding an exact result to bf16 is 1.7e-3)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import bsattn_oracle as orc
+from helpers import make_qkv, uniform_block_mask, causal_block_mask, errors, f32
+
+pytestmark = pytest.mark.gpu
+
+MAXABS = {torch.float16: 2e-2, torch.bfloat16: 3e-2}
+RELL2 = 1e-3
+
+
+def run_case(dev, B, H, N, D, dtype, mask, seed, out_fp32=False, check_lse=True):
+    import fa2_custom_mask as fm
+    q, k, v = make_qkv(B, H, N, D, dtype, seed)
+    sm_scale = 1.0 / np.sqrt(D)
+    o_ref, lse_ref = orc.naive_attention(f32(q), f32(k), f32(v), mask.numpy(), sm_scale, return_lse=True)
+    o, lse = fm.flash_attention_custom_mask_lse(q.to(dev), k.to(dev), v.to(dev), mask.to(dev), sm_scale,
+                                                out_fp32=out_fp32)
+    torch.cuda.synchronize()
+    assert o.dtype == (torch.float32 if out_fp32 else dtype) and tuple(o.shape) == (B, H, N, D)
+    ma, rl = errors(o, o_ref)
+    print("B%d H%d N%d D%d %s fp32out=%s: max-abs %.3e rel-L2 %.3e" % (B, H, N, D, dtype, out_fp32, ma, rl))
+    assert ma <= MAXABS[dtype]
+    if dtype == torch.float16 or out_fp32:
+        assert rl <= RELL2
+    else:
+        assert rl <= 3e-3          # bf16-typed output: the cast alone costs 1.7e-3
+    if check_lse:
+        fin = np.isfinite(lse_ref)
+        l = lse.cpu().numpy()
+        assert np.array_equal(np.isfinite(l), fin)
+        assert np.abs(l[fin] - lse_ref[fin]).max() <= 2e-3
+    return o
+
+
+def test_c1_config(dev):
+    """B=1 H=1 N=1024 D=64, 16x16 tiles kept with p=0.5 + diagonal."""
+    run_case(dev, 1, 1, 1024, 64, torch.float16, uniform_block_mask(1, 1, 16, 0.5, 1234), 1234)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [64, 128])
+def test_small_shapes(dev, D, dtype):
+    run_case(dev, 2, 3, 512, D, dtype, uniform_block_mask(2, 3, 8, 0.4, 5), 17)
+    run_case(dev, 2, 3, 512, D, dtype, uniform_block_mask(2, 3, 8, 0.4, 5), 17, out_fp32=True)
+
+
+def test_shared_mask_broadcast(dev):
+    m = causal_block_mask(1, 1, 12, 0.5, 9)
+    run_case(dev, 2, 4, 768, 64, torch.float16, m, 3)
+    run_case(dev, 2, 4, 768, 64, torch.float16, uniform_block_mask(2, 1, 12, 0.3, 4), 3)
+    run_case(dev, 2, 4, 768, 64, torch.float16, uniform_block_mask(1, 4, 12, 0.3, 4), 3)
+
+
+def test_empty_rows_and_all_false(dev):
+    import fa2_custom_mask as fm
+    m = uniform_block_mask(1, 2, 8, 0.3, 2)
+    m[0, 0, 3, :] = False
+    m[0, 1, 0, :] = False
+    o = run_case(dev, 1, 2, 512, 64, torch.float16, m, 8)
+    assert float(o[0, 0, 192:256].abs().max()) == 0.0 and float(o[0, 1, 0:64].abs().max()) == 0.0
+    q, k, v = [x.to(dev) for x in make_qkv(1, 2, 512, 64, torch.float16, 8)]
+    z = fm.flash_attention_custom_mask(q, k, v, torch.zeros(1, 2, 8, 8, dtype=torch.bool, device=dev), 0.125)
+    assert float(z.abs().max()) == 0.0                                       # fa2_custom_mask.py:49-51
+
+
+def test_dense_elementwise_mask_c2_small(dev):
+    """Tile-constant elementwise mask gives the same result as its block mask."""
+    import fa2_custom_mask as fm
+    N, D = 1280, 64
+    block = uniform_block_mask(1, 1, N // 64, 0.3, 6)
+    q, k, v = [x.to(dev) for x in make_qkv(1, 1, N, D, torch.float16, 6)]
+    dense = block.to(dev).repeat_interleave(64, 2).repeat_interleave(64, 3)
+    o1 = fm.flash_attention_custom_mask(q, k, v, block.to(dev), 0.125)
+    o2 = fm.flash_attention_custom_mask(q, k, v, dense, 0.125)
+    assert torch.equal(o1, o2)
+
+
+def test_strided_inputs(dev):
+    import fa2_custom_mask as fm
+    B, H, N, D = 1, 2, 512, 64
+    g = torch.Generator().manual_seed(0)
+    qkv = torch.randn(B, N, 3, H, D, generator=g).to(torch.float16).to(dev)  # packed layout
+    q, k, v = [qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3)]
+    m = uniform_block_mask(1, 1, 8, 0.5, 1).to(dev)
+    o1 = fm.flash_attention_custom_mask(q, k, v, m, 0.125)
+    o2 = fm.flash_attention_custom_mask(q.contiguous(), k.contiguous(), v.contiguous(), m, 0.125)
+    assert torch.equal(o1, o2)
+
+
+@pytest.mark.parametrize("keep", [0.1, 1.0])
+def test_c2_config(dev, keep):
+    """N=6400 D=64 fp16, 100x100 tiles."""
+    run_case(dev, 1, 1, 6400, 64, torch.float16, uniform_block_mask(1, 1, 100, keep, 1235), 1235)
+
+
+def test_determinism(dev):
+    import fa2_custom_mask as fm
+    q, k, v = [x.to(dev) for x in make_qkv(1, 2, 2048, 64, torch.float16, 5)]
+    m = uniform_block_mask(1, 2, 32, 0.3, 5).to(dev)
+    o1 = fm.flash_attention_custom_mask(q, k, v, m, 0.125)
+    o2 = fm.flash_attention_custom_mask(q, k, v, m, 0.125)
+    assert torch.equal(o1, o2)
+
+
+def test_invariants_large(dev):
+    """Size-independent properties at the headline size N=17536: v = 1 gives O = 1, and
+    k = 0 gives the mean of the kept V rows."""
+    import fa2_custom_mask as fm
+    N, D, nb = 17536, 64, 274
+    q, k, v = [x.to(dev) for x in make_qkv(1, 1, N, D, torch.float16, 77)]
+    m = uniform_block_mask(1, 1, nb, 0.1, 77).to(dev)
+    o = fm.flash_attention_custom_mask(q, k, torch.ones_like(v), m, 0.125)
+    assert float((o.float() - 1).abs().max()) <= 2e-3
+    o = fm.flash_attention_custom_mask(q, torch.zeros_like(k), v, m, 0.125)
+    mean = torch.zeros(N, D, device=dev)
+    vt = v[0, 0].float().view(nb, 64, D).mean(1)                              # per-tile means
+    w = m[0, 0].float()
+    mean_rows = (w @ vt) / w.sum(1, keepdim=True)
+    ref = mean_rows.repeat_interleave(64, 0)
+    assert float((o[0, 0].float() - ref).abs().max()) <= 2e-3
