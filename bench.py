@@ -1,0 +1,150 @@
+#!/usr/bin/env python3
+"""Benchmark of the block-sparse attention forward on one MI355X.
+
+Workload (BASELINE.json configs[2]): forward, B=1 H=1 N=17536 D=64 fp16, 274x274 tile grid,
+kept-tile ratios {0.05, 0.1, 0.25, 0.5, 1.0} (random tiles + forced diagonal), kernel time
+measured separately from mask preprocessing.  One "step" is one forward pass at keep 1.0 with
+q/k/v and the kept-tile lists already resident in HBM.  Prints one JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "customize-block-sparse-attention-with-triton_amd"))
+sys.path.insert(0, ROOT)
+
+N, D, TILE = 17536, 64, 64
+NB = N // TILE
+KEEPS = [0.05, 0.1, 0.25, 0.5, 1.0]
+PEAK_F16_TFLOPS = 2500.0     # MI355X dense fp16 MFMA
+PEAK_HBM_GBS = 8000.0
+SEED = 1234 + 2
+
+
+def tile_flops(kept):
+    return kept * 4.0 * TILE * TILE * D          # QK^T + PV per kept tile
+
+
+def event_times(fn, iters, warmup, torch):
+    for _ in range(warmup):
+        fn()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return sorted(a.elapsed_time(b) for a, b in evs)       # ms
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (heads / row blocks shard without "
+              "communication; no multi-GPU figure is produced). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    import fa2_custom_mask as fm
+    from fa2_custom_mask import fa2_custom_mask as host
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(SEED)
+    q, k, v = [torch.randn(1, 1, N, D, generator=g).to(torch.float16) for _ in range(3)]
+    masks = {}
+    for r in KEEPS:
+        m = torch.rand(1, 1, NB, NB, generator=g) < r
+        masks[r] = m | torch.eye(NB, dtype=torch.bool)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    sm_scale = 1.0 / np.sqrt(D)
+
+    lists = {r: fm.block_mask_to_lists(masks[r].to(dev)) for r in KEEPS}
+    kept = {r: int(lists[r].counts[1]) for r in KEEPS}
+
+    def fwd(r):
+        return host._forward(qd, kd, vd, lists[r], sm_scale, torch.float16, True)
+
+    # ---- headline: K timed steps at keep 1.0 ----
+    for _ in range(args.warmup):
+        fwd(1.0)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        fwd(1.0)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    value = tile_flops(kept[1.0]) / (ms_per_step * 1e-3) / 1e12
+
+    # ---- per-launch device time (HIP events on the launch stream), sweep of kept ratios ----
+    sweep = {}
+    for r in KEEPS:
+        ts = event_times(lambda: fwd(r), max(20, args.steps), 5, torch)
+        avg, med = sum(ts) / len(ts), ts[len(ts) // 2]
+        sweep[str(r)] = {"kept_tiles": kept[r], "ms_avg": round(avg, 5), "ms_median": round(med, 5),
+                         "tflops": round(tile_flops(kept[r]) / (med * 1e-3) / 1e12, 2),
+                         "frac_mfma_peak": round(tile_flops(kept[r]) / (med * 1e-3) / 1e12 / PEAK_F16_TFLOPS, 4)}
+    dense_avg_ms = sweep["1.0"]["ms_avg"]
+    achieved = tile_flops(kept[1.0]) / (dense_avg_ms * 1e-3) / 1e12
+    ratio = sweep["0.1"]["ms_median"] / sweep["1.0"]["ms_median"]
+
+    # ---- mask preprocessing: dense N x N bool -> block mask -> lists (HBM bound) ----
+    dense_mask = masks[0.1].to(dev).repeat_interleave(TILE, 2).repeat_interleave(TILE, 3)
+    ts = event_times(lambda: fm.block_mask_to_lists(fm.reduce_dense_mask(dense_mask)), 20, 3, torch)
+    pre_ms = ts[len(ts) // 2]
+    pre_bytes = float(N) * N + 4.0 * (kept[0.1] + 5 * NB)
+    ts_b = event_times(lambda: fm.block_mask_to_lists(masks[0.1].to(dev)), 20, 3, torch)
+    del dense_mask
+
+    # ---- parity spot check against the CPU oracle (first 2 row blocks, keep 0.1) ----
+    from oracle import c_oracle
+    o_gpu, _ = fwd(0.1)
+    o_ref, _ = c_oracle.naive_fwd(q.float().numpy(), k.float().numpy(), v.float().numpy(),
+                                  masks[0.1].numpy(), sm_scale, 0, 128)
+    parity = float(np.abs(o_gpu[0, 0, :128].float().cpu().numpy() - o_ref[0, 0, :128]).max())
+
+    out = {
+        "metric": "fwd effective TFLOP/s on kept tiles, N=17536 D=64 fp16, keep 1.0 (kernel only)",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "BASELINE configs[2]: fwd B=1 H=1 N=17536 D=64 fp16, 274x274 tiles, keep 1.0",
+                   "kept_tiles": kept[1.0], "seed": SEED},
+        "sweep": sweep,
+        "keep0.1_over_keep1.0_time": round(ratio, 4),
+        "mask_preprocess": {"dense_NxN_ms": round(pre_ms, 5), "dense_GBps": round(pre_bytes / (pre_ms * 1e-3) / 1e9, 1),
+                            "frac_hbm_peak": round(pre_bytes / (pre_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                            "block_mask_ms": round(ts_b[len(ts_b) // 2], 5)},
+        "parity_max_abs_vs_oracle": parity,
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": None,
+                     "kernel": "fwd_kernel<64,false> + combine_kernel<64,false> (one bsattn_fwd call)"},
+    }
+    if not args.no_cpu:
+        # CPU baseline: the oracle's C port of the naive path, all host threads, on the first
+        # 4096 query rows of the same keep-1.0 workload (every key), reported in the metric's unit.
+        rows = 4096
+        qf, kf, vf = q.float().numpy(), k.float().numpy(), v.float().numpy()
+        c_oracle.naive_fwd(qf, kf, vf, masks[1.0].numpy(), sm_scale, 0, 64)
+        t0 = time.perf_counter()
+        c_oracle.naive_fwd(qf, kf, vf, masks[1.0].numpy(), sm_scale, 0, rows)
+        dt = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": round(4.0 * rows * N * D / dt / 1e12, 5), "unit": "TFLOP/s",
+                               "cores": c_oracle.num_threads(), "kind": "port",
+                               "sample": "first %d of %d query rows, all keys, keep 1.0, fp32 naive "
+                                         "masked softmax (oracle C port, OpenMP), %.2f s" % (rows, N, dt)}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
