@@ -14,7 +14,8 @@ struct HeadSplit {
 };
 
 // rp: row pointers of the head (nb + 1 entries, absolute offsets)
-__device__ __forceinline__ HeadSplit head_split(const int32_t* rp, int nb, int P) {
+template <typename Ptr>
+__device__ __forceinline__ HeadSplit head_split(Ptr rp, int nb, int P) {
   HeadSplit s;
   s.lo = rp[0];
   s.T = rp[nb] - s.lo;
