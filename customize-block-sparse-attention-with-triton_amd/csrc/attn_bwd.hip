@@ -1,7 +1,398 @@
+// Block-sparse FlashAttention-2 backward for gfx950.
+//
+// Gradient algebra of the reference (fa2_custom_mask/fa2_bwd.py:17,57-74,117-130,232,284),
+// evaluated over exactly the kept tiles:
+//   delta = rowsum(O * dO);  P = exp(S*sm_scale - lse);  dV = P^T dO;  dP = dO V^T;
+//   dS = P * (dP - delta);   dK = sm_scale * dS^T Q;     dQ = sm_scale * dS K.
+// Three kernels, no atomics, results independent of scheduling:
+//   delta_kernel  one pass over O and dO (HBM bound);
+//   dq_kernel     one workgroup (2 wavefronts x 32 queries) per row block, walking the row
+//                 lists: per kept tile  S^T = K Q^T,  dP^T = V dO^T,  dQ^T += K^T dS^T;
+//   dkdv_kernel   one workgroup (2 wavefronts x 32 keys) per column block, walking the column
+//                 lists: per kept tile  S = Q K^T,  dP = dO V^T,  dV^T += dO^T P,  dK^T += Q^T dS.
+// Operand roles are chosen so that the fragment a wavefront owns for the whole walk (Q, dO or
+// K, V) sits along the lanes: the per-row scalars (lse, delta) are then per-lane values in
+// dq_kernel, P and dS leave the first products already in the operand layout of the second
+// ones, and the tiles that change per step are staged in LDS by asynchronous copies into a
+// double buffer (one barrier per tile).
 #include "common.h"
+#include "kernel_util.h"
+
 namespace bsattn {
-size_t bwd_workspace_bytes(int B, int H, int N, int D) { return 256; }
-int launch_bwd(const void*, const void*, const void*, const void*, const void*, const float*, void*, void*,
-               void*, const int32_t*, const int32_t*, const int32_t*, const int32_t*, const AttnShape&,
-               void*, hipStream_t) { return BSATTN_ERR_LAUNCH; }
+
+struct BwdParams {
+  const void* q; const void* k; const void* v; const void* o; const void* d_o;
+  const float* lse; float* delta;
+  void* dq; void* dk; void* dv;
+  const int32_t* row_ptr; const int32_t* col_idx; const int32_t* col_ptr; const int32_t* row_idx;
+  int B, H, N, nb, Bm, Hm;
+  int out_f32;
+  float sm_scale, qk_scale;   // qk_scale = sm_scale * log2(e)
+  int64_t qs[3], ks[3], vs[3], os[3], dos[3];
+};
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+// ---------------------------------------------------------------------------------------
+// delta[b,h,n] = sum_d O[n,d] * dO[n,d]   (fa2_bwd.py:17).  8 (D=64) or 16 (D=128) lanes per row.
+// ---------------------------------------------------------------------------------------
+template <int D, bool BF16>
+__global__ __launch_bounds__(256) void delta_kernel(const BwdParams prm) {
+  constexpr int LPR = D / 8;            // lanes per row, 16 bytes each
+  constexpr int RPB = 256 / LPR;        // rows per workgroup
+  const int bh = blockIdx.y, b = bh / prm.H, h = bh % prm.H;
+  const int row = blockIdx.x * RPB + threadIdx.x / LPR, part = threadIdx.x % LPR;
+  if (row >= prm.N) return;
+  const unsigned short* op = (const unsigned short*)prm.o + b * prm.os[0] + h * prm.os[1] + (int64_t)row * prm.os[2] + part * 8;
+  const unsigned short* gp = (const unsigned short*)prm.d_o + b * prm.dos[0] + h * prm.dos[1] + (int64_t)row * prm.dos[2] + part * 8;
+  const uintx4 ov = *reinterpret_cast<const uintx4*>(op);
+  const uintx4 gv = *reinterpret_cast<const uintx4*>(gp);
+  float acc = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    float o0, o1, g0, g1;
+    const unsigned int ou = ov[i], gu = gv[i];   // by value: bit_cast of a vector element lvalue miscompiles
+    if constexpr (BF16) {
+      o0 = __builtin_bit_cast(float, ou << 16); o1 = __builtin_bit_cast(float, ou & 0xffff0000u);
+      g0 = __builtin_bit_cast(float, gu << 16); g1 = __builtin_bit_cast(float, gu & 0xffff0000u);
+    } else {
+      const half2v oh = __builtin_bit_cast(half2v, ou), gh = __builtin_bit_cast(half2v, gu);
+      o0 = (float)oh[0]; o1 = (float)oh[1]; g0 = (float)gh[0]; g1 = (float)gh[1];
+    }
+    acc += o0 * g0 + o1 * g1;
+  }
+#pragma unroll
+  for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+  if (part == 0) prm.delta[(int64_t)bh * prm.N + row] = acc;
 }
+
+// ---------------------------------------------------------------------------------------
+// helpers of the two walking kernels
+// ---------------------------------------------------------------------------------------
+template <int D> struct BwdCfg {
+  static constexpr int TILE_BYTES = 64 * 2 * D;
+  static constexpr int STAT_BYTES = 2 * 64 * 4;                    // lse2[64] + delta[64] of a row block
+  static constexpr int STAGE_BYTES = 2 * TILE_BYTES + STAT_BYTES;  // two tiles (+ row statistics)
+  static constexpr int LDS_BYTES = 2 * STAGE_BYTES;                // double buffer
+};
+
+// This wavefront's half of the asynchronous copy of a 64 x D tile (rows `stride` elements apart)
+// into LDS with the u_swz chunk swizzle: wavefront wv issues instructions [wv*D/16, (wv+1)*D/16).
+template <int D>
+__device__ __forceinline__ void half_tile_load_async(const unsigned short* tile, int64_t stride, int wv, int lane,
+                                                     unsigned lds_addr) {
+  constexpr int CPR = D / 8;
+#pragma unroll
+  for (int jj = 0; jj < CPR / 2; ++jj) {
+    const int j = wv * (CPR / 2) + jj;
+    const int c = j * 64 + lane, row = c / CPR, ch = c % CPR;
+    const unsigned off = 2u * (unsigned)(row * (int)stride + ((ch ^ u_swz<D>(row)) * 8));
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_addr + j * 1024), "v"(off), "s"(tile) : "memory", "m0");
+  }
+}
+
+// asynchronous copy of 64 consecutive floats (one per lane)
+__device__ __forceinline__ void stat_load_async(const float* src, int lane, unsigned lds_addr) {
+  const unsigned off = 4u * (unsigned)lane;
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2" :: "s"(lds_addr), "v"(off), "s"(src) : "memory", "m0");
+}
+
+// operand fragment (32 rows x 16 columns slice s) of a swizzled LDS tile: row r0 + ln, chunk 2s + g
+template <int D>
+__device__ __forceinline__ uintx4 frag_rows(const unsigned char* tile, int r0, int s, int ln, int g) {
+  const int row = r0 + ln;
+  return *reinterpret_cast<const uintx4*>(tile + row * 2 * D + (((2 * s + g) ^ u_swz<D>(row)) * 16));
+}
+
+// transposed operand fragment: columns 32db + ln of the tile along the lanes, contraction slots j
+// of slice ts <-> tile rows 16ts + 8(j/4) + 4g + (j%4) (the order in which a 32x32 MFMA result
+// holds its rows), by two LDS transpose reads
+template <int D, bool BF16>
+__device__ __forceinline__ uintx4 frag_cols(const unsigned char* tile, int db, int ts, int lane) {
+  const int blk = lane >> 4, s16 = lane & 15;
+  uintx4 a;
+#pragma unroll
+  for (int jh = 0; jh < 2; ++jh) {
+    const int row = 16 * ts + 8 * jh + 4 * (blk >> 1) + (s16 >> 2);
+    const int col = 32 * db + 16 * (blk & 1) + 4 * (s16 & 3);
+    const int addr = row * 2 * D + (((col >> 3) ^ u_swz<D>(row)) * 16) + (col & 7) * 2;
+    const short4v rr = __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4v __attribute__((address_space(3)))*)(tile + addr));
+    const uintx2 r2 = __builtin_bit_cast(uintx2, rr);
+    a[2 * jh] = r2[0]; a[2 * jh + 1] = r2[1];
+  }
+  if constexpr (BF16) a = bf16x8_to_f16x8(a);
+  return a;
+}
+
+__device__ __forceinline__ floatx16 mfma_f16(uintx4 a, uintx4 b, floatx16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ unsigned int pack_half2(float a, float b) {
+  const half2v h = {(_Float16)a, (_Float16)b};
+  return __builtin_bit_cast(unsigned int, h);
+}
+
+__device__ __forceinline__ floatx16 zero16() {
+  floatx16 z;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) z[i] = 0.f;
+  return z;
+}
+
+// ---------------------------------------------------------------------------------------
+// dQ: workgroup = row block m, wavefront wv owns queries 64m + 32wv + ln
+// ---------------------------------------------------------------------------------------
+template <int D, bool BF16>
+__global__ __launch_bounds__(128) void dq_kernel(const BwdParams prm) {
+  using C = BwdCfg<D>;
+  constexpr int KS = D / 16, DB = D / 32;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+  const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int ln = lane & 31, g = lane >> 5;
+  const int nb = prm.nb;
+  const int m = nb - 1 - blockIdx.x;          // long rows of block-causal masks first
+  const int bh = blockIdx.y, b = bh / prm.H, h = bh % prm.H;
+  const int mh = (prm.Bm > 1 ? b : 0) * prm.Hm + (prm.Hm > 1 ? h : 0);
+  const cint_ptr_t rp = (cint_ptr_t)(uintptr_t)(prm.row_ptr + (int64_t)mh * nb);
+  const cint_ptr_t cols = (cint_ptr_t)(uintptr_t)prm.col_idx;
+  const int t0 = rp[m], t1 = rp[m + 1];
+  const unsigned lds_addr = (unsigned)(uintptr_t)(lds_ptr_t)lds;
+
+  const unsigned short* kg = (const unsigned short*)prm.k + b * prm.ks[0] + h * prm.ks[1];
+  const unsigned short* vg = (const unsigned short*)prm.v + b * prm.vs[0] + h * prm.vs[1];
+  auto issue = [&](int t, int stage) {
+    const int cb = cols[t];
+    half_tile_load_async<D>(kg + (int64_t)cb * 64 * prm.ks[2], prm.ks[2], wv, lane, lds_addr + stage * C::STAGE_BYTES);
+    half_tile_load_async<D>(vg + (int64_t)cb * 64 * prm.vs[2], prm.vs[2], wv, lane,
+                            lds_addr + stage * C::STAGE_BYTES + C::TILE_BYTES);
+  };
+  if (t0 < t1) issue(t0, 0);
+
+  const int64_t qrow = (int64_t)m * 64 + 32 * wv + ln;
+  const unsigned short* qp = (const unsigned short*)prm.q + b * prm.qs[0] + h * prm.qs[1] + qrow * prm.qs[2];
+  const unsigned short* gp = (const unsigned short*)prm.d_o + b * prm.dos[0] + h * prm.dos[1] + qrow * prm.dos[2];
+  uintx4 qfr[KS], dofr[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    qfr[s] = *reinterpret_cast<const uintx4*>(qp + 16 * s + 8 * g);
+    dofr[s] = *reinterpret_cast<const uintx4*>(gp + 16 * s + 8 * g);
+  }
+  const float lse2 = prm.lse[(int64_t)bh * prm.N + qrow] * kLog2e;
+  const float dlt = prm.delta[(int64_t)bh * prm.N + qrow];
+  // compiler-visible vmcnt(0): everything above has arrived, no vector-memory waits in the loop
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+  const float qk_scale = prm.qk_scale;
+
+  floatx16 dqacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) dqacc[db] = zero16();
+
+  for (int t = t0; t < t1; ++t) {
+    const int stage = (t - t0) & 1;
+    wait_vm<0>();
+    __syncthreads();   // tile t complete in `stage`; everyone is done with the other stage
+    if (t + 1 < t1) issue(t + 1, stage ^ 1);
+    const unsigned char* kt = lds + stage * C::STAGE_BYTES;
+    const unsigned char* vt = kt + C::TILE_BYTES;
+
+    floatx16 sacc[2], dpacc[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) { sacc[kb] = zero16(); dpacc[kb] = zero16(); }
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        sacc[kb] = mfma_qk<BF16>(frag_rows<D>(kt, 32 * kb, s, ln, g), qfr[s], sacc[kb]);      // S^T = K Q^T
+        dpacc[kb] = mfma_qk<BF16>(frag_rows<D>(vt, 32 * kb, s, ln, g), dofr[s], dpacc[kb]);   // dP^T = V dO^T
+      }
+    // dS^T = P^T * (dP^T - delta), this lane's query; packed as operand slices of 16 keys
+    uintx4 dsf[4];
+#pragma unroll
+    for (int ts = 0; ts < 4; ++ts)
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        const int kb = ts >> 1, i = 8 * (ts & 1) + 2 * jj;
+        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][i], qk_scale, -lse2));
+        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][i + 1], qk_scale, -lse2));
+        dsf[ts][jj] = pack_half2(p0 * (dpacc[kb][i] - dlt), p1 * (dpacc[kb][i + 1] - dlt));
+      }
+#pragma unroll
+    for (int ts = 0; ts < 4; ++ts)
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+        dqacc[db] = mfma_f16(frag_cols<D, BF16>(kt, db, ts, lane), dsf[ts], dqacc[db]);          // dQ^T += K^T dS^T
+  }
+
+  void* base = prm.out_f32 ? (void*)((float*)prm.dq + (int64_t)bh * prm.N * D) : (void*)((unsigned short*)prm.dq + (int64_t)bh * prm.N * D);
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4)
+      store_out4<BF16>(base, qrow * D + 32 * db + 8 * i4 + 4 * g, prm.out_f32, dqacc[db][4 * i4] * prm.sm_scale,
+                       dqacc[db][4 * i4 + 1] * prm.sm_scale, dqacc[db][4 * i4 + 2] * prm.sm_scale,
+                       dqacc[db][4 * i4 + 3] * prm.sm_scale);
+}
+
+// ---------------------------------------------------------------------------------------
+// dK, dV: workgroup = column block n, wavefront wv owns keys 64n + 32wv + ln
+// ---------------------------------------------------------------------------------------
+template <int D, bool BF16>
+__global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
+  using C = BwdCfg<D>;
+  constexpr int KS = D / 16, DB = D / 32;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+  const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int ln = lane & 31, g = lane >> 5;
+  const int nb = prm.nb;
+  const int n = blockIdx.x;                   // early columns of block-causal masks are the long ones
+  const int bh = blockIdx.y, b = bh / prm.H, h = bh % prm.H;
+  const int mh = (prm.Bm > 1 ? b : 0) * prm.Hm + (prm.Hm > 1 ? h : 0);
+  const cint_ptr_t cp = (cint_ptr_t)(uintptr_t)(prm.col_ptr + (int64_t)mh * nb);
+  const cint_ptr_t rows = (cint_ptr_t)(uintptr_t)prm.row_idx;
+  const int t0 = cp[n], t1 = cp[n + 1];
+  const unsigned lds_addr = (unsigned)(uintptr_t)(lds_ptr_t)lds;
+
+  const unsigned short* qg = (const unsigned short*)prm.q + b * prm.qs[0] + h * prm.qs[1];
+  const unsigned short* gg = (const unsigned short*)prm.d_o + b * prm.dos[0] + h * prm.dos[1];
+  const float* lse_h = prm.lse + (int64_t)bh * prm.N;
+  const float* dlt_h = prm.delta + (int64_t)bh * prm.N;
+  auto issue = [&](int t, int stage) {
+    const int rb = rows[t];
+    const unsigned sa = lds_addr + stage * C::STAGE_BYTES;
+    half_tile_load_async<D>(qg + (int64_t)rb * 64 * prm.qs[2], prm.qs[2], wv, lane, sa);
+    half_tile_load_async<D>(gg + (int64_t)rb * 64 * prm.dos[2], prm.dos[2], wv, lane, sa + C::TILE_BYTES);
+    stat_load_async((wv == 0 ? lse_h : dlt_h) + rb * 64, lane, sa + 2 * C::TILE_BYTES + wv * 256);
+  };
+  if (t0 < t1) issue(t0, 0);
+
+  const int64_t krow = (int64_t)n * 64 + 32 * wv + ln;
+  const unsigned short* kp = (const unsigned short*)prm.k + b * prm.ks[0] + h * prm.ks[1] + krow * prm.ks[2];
+  const unsigned short* vp = (const unsigned short*)prm.v + b * prm.vs[0] + h * prm.vs[1] + krow * prm.vs[2];
+  uintx4 kfr[KS], vfr[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    kfr[s] = *reinterpret_cast<const uintx4*>(kp + 16 * s + 8 * g);
+    vfr[s] = *reinterpret_cast<const uintx4*>(vp + 16 * s + 8 * g);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // compiler-visible vmcnt(0), as in dq_kernel
+  const float qk_scale = prm.qk_scale;
+
+  floatx16 dkacc[DB], dvacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) { dkacc[db] = zero16(); dvacc[db] = zero16(); }
+
+  for (int t = t0; t < t1; ++t) {
+    const int stage = (t - t0) & 1;
+    wait_vm<0>();
+    __syncthreads();
+    if (t + 1 < t1) issue(t + 1, stage ^ 1);
+    const unsigned char* qt = lds + stage * C::STAGE_BYTES;
+    const unsigned char* gt = qt + C::TILE_BYTES;
+    const float* st_lse = reinterpret_cast<const float*>(gt + C::TILE_BYTES);
+    const float* st_dlt = st_lse + 64;
+
+    floatx16 sacc[2], dpacc[2];
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) { sacc[qb] = zero16(); dpacc[qb] = zero16(); }
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) {
+        sacc[qb] = mfma_qk<BF16>(frag_rows<D>(qt, 32 * qb, s, ln, g), kfr[s], sacc[qb]);      // S = Q K^T
+        dpacc[qb] = mfma_qk<BF16>(frag_rows<D>(gt, 32 * qb, s, ln, g), vfr[s], dpacc[qb]);    // dP = dO V^T
+      }
+    // rows of the results are queries: register i of block qb <-> query 32qb + 8(i/4) + 4g + i%4
+    uintx4 pf[4], dsf[4];
+#pragma unroll
+    for (int ts = 0; ts < 4; ++ts)
+#pragma unroll
+      for (int jh = 0; jh < 2; ++jh) {
+        const int qb = ts >> 1, i0 = 8 * (ts & 1) + 4 * jh;
+        const int q0 = 32 * qb + 8 * (i0 >> 2) + 4 * g;
+        const floatx4 l4 = *reinterpret_cast<const floatx4*>(st_lse + q0);
+        const floatx4 d4 = *reinterpret_cast<const floatx4*>(st_dlt + q0);
+        float p[4], ds[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[qb][i0 + e], qk_scale, -l4[e] * kLog2e));
+          ds[e] = p[e] * (dpacc[qb][i0 + e] - d4[e]);
+        }
+        pf[ts][2 * jh] = pack_half2(p[0], p[1]);   pf[ts][2 * jh + 1] = pack_half2(p[2], p[3]);
+        dsf[ts][2 * jh] = pack_half2(ds[0], ds[1]); dsf[ts][2 * jh + 1] = pack_half2(ds[2], ds[3]);
+      }
+#pragma unroll
+    for (int ts = 0; ts < 4; ++ts)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        dvacc[db] = mfma_f16(frag_cols<D, BF16>(gt, db, ts, lane), pf[ts], dvacc[db]);    // dV^T += dO^T P
+        dkacc[db] = mfma_f16(frag_cols<D, BF16>(qt, db, ts, lane), dsf[ts], dkacc[db]);   // dK^T += Q^T dS
+      }
+  }
+
+  const int64_t hoff = (int64_t)bh * prm.N * D;
+  void* kbase = prm.out_f32 ? (void*)((float*)prm.dk + hoff) : (void*)((unsigned short*)prm.dk + hoff);
+  void* vbase = prm.out_f32 ? (void*)((float*)prm.dv + hoff) : (void*)((unsigned short*)prm.dv + hoff);
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) {
+      const int64_t off = krow * D + 32 * db + 8 * i4 + 4 * g;
+      store_out4<BF16>(kbase, off, prm.out_f32, dkacc[db][4 * i4] * prm.sm_scale, dkacc[db][4 * i4 + 1] * prm.sm_scale,
+                       dkacc[db][4 * i4 + 2] * prm.sm_scale, dkacc[db][4 * i4 + 3] * prm.sm_scale);
+      store_out4<BF16>(vbase, off, prm.out_f32, dvacc[db][4 * i4], dvacc[db][4 * i4 + 1], dvacc[db][4 * i4 + 2],
+                       dvacc[db][4 * i4 + 3]);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------
+size_t bwd_workspace_bytes(int B, int H, int N, int D) {
+  (void)D;
+  return (size_t)B * H * N * sizeof(float);   // delta
+}
+
+template <int D, bool BF16>
+static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
+  using C = BwdCfg<D>;
+  static bool configured = false;   // raising the dynamic LDS limit is idempotent
+  if (!configured) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dq_kernel<D, BF16>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv_kernel<D, BF16>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+    configured = true;
+  }
+  const int BH = prm.B * prm.H;
+  constexpr int RPB = 256 / (D / 8);
+  hipLaunchKernelGGL((delta_kernel<D, BF16>), dim3((prm.N + RPB - 1) / RPB, BH), dim3(256), 0, st, prm);
+  hipLaunchKernelGGL((dq_kernel<D, BF16>), dim3(prm.nb, BH), dim3(128), C::LDS_BYTES, st, prm);
+  hipLaunchKernelGGL((dkdv_kernel<D, BF16>), dim3(prm.nb, BH), dim3(128), C::LDS_BYTES, st, prm);
+}
+
+int launch_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
+               const float* lse, void* dq, void* dk, void* dv, const int32_t* row_ptr,
+               const int32_t* col_idx, const int32_t* col_ptr, const int32_t* row_idx,
+               const AttnShape& s, void* ws, hipStream_t st) {
+  BwdParams prm;
+  prm.q = q; prm.k = k; prm.v = v; prm.o = o; prm.d_o = d_o; prm.lse = lse; prm.delta = (float*)ws;
+  prm.dq = dq; prm.dk = dk; prm.dv = dv;
+  prm.row_ptr = row_ptr; prm.col_idx = col_idx; prm.col_ptr = col_ptr; prm.row_idx = row_idx;
+  prm.B = s.B; prm.H = s.H; prm.N = s.N; prm.nb = s.N / 64; prm.Bm = s.Bm; prm.Hm = s.Hm;
+  prm.out_f32 = s.out_dtype == BSATTN_F32;
+  prm.sm_scale = s.sm_scale;
+  prm.qk_scale = s.sm_scale * kLog2e;
+  for (int i = 0; i < 3; ++i) {
+    prm.qs[i] = s.qs[i]; prm.ks[i] = s.ks[i]; prm.vs[i] = s.vs[i]; prm.os[i] = s.os[i]; prm.dos[i] = s.dos[i];
+  }
+  const bool bf = s.dtype == BSATTN_BF16;
+  if (s.D == 64 && !bf) launch_bwd_t<64, false>(prm, st);
+  else if (s.D == 64 && bf) launch_bwd_t<64, true>(prm, st);
+  else if (s.D == 128 && !bf) launch_bwd_t<128, false>(prm, st);
+  else launch_bwd_t<128, true>(prm, st);
+  return launch_status();
+}
+
+}  // namespace bsattn

@@ -5,7 +5,6 @@
 
 namespace bsattn {
 
-constexpr int kMinTilesPerRange = 4;  // do not cut a head into ranges shorter than this
 
 struct HeadSplit {
   int lo;    // first tile of the head in the global list
@@ -15,11 +14,11 @@ struct HeadSplit {
 
 // rp: row pointers of the head (nb + 1 entries, absolute offsets)
 template <typename Ptr>
-__device__ __forceinline__ HeadSplit head_split(Ptr rp, int nb, int P) {
+__device__ __forceinline__ HeadSplit head_split(Ptr rp, int nb, int P, int min_tiles) {
   HeadSplit s;
   s.lo = rp[0];
   s.T = rp[nb] - s.lo;
-  const int want = (s.T + kMinTilesPerRange - 1) / kMinTilesPerRange;
+  const int want = (s.T + min_tiles - 1) / min_tiles;   // no range shorter than min_tiles
   s.Peff = want < P ? want : P;
   return s;
 }

@@ -1,0 +1,125 @@
+// Device-side helpers shared by the attention kernels: vector types, MFMA wrappers, LDS tile
+// swizzles, asynchronous global->LDS tile copies and output stores.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace bsattn {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short short8 __attribute__((ext_vector_type(8)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
+typedef unsigned int uintx2 __attribute__((ext_vector_type(2)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+
+
+__device__ __forceinline__ float max3f(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
+__device__ __forceinline__ float xhalf_max(float x) {
+  // max of lane l and lane l^32 (the two halves of a wavefront hold the same query)
+  return fmaxf(x, __shfl_xor(x, 32));
+}
+
+template <bool BF16>
+__device__ __forceinline__ floatx16 mfma_qk(uintx4 a, uintx4 b, floatx16 c) {
+  if constexpr (BF16)
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a),
+                                                  __builtin_bit_cast(half8, b), c, 0, 0, 0);
+}
+
+// two packed fp16 values times an fp32 scalar, rounded back to fp16
+__device__ __forceinline__ unsigned int scale_half2(unsigned int x, float c) {
+  const half2v h = __builtin_bit_cast(half2v, x);
+  const half2v r = {(_Float16)((float)h[0] * c), (_Float16)((float)h[1] * c)};
+  return __builtin_bit_cast(unsigned int, r);
+}
+
+// bf16 bits -> fp16 bits, 8 at a time (exact for the magnitudes attention inputs take)
+__device__ __forceinline__ uintx4 bf16x8_to_f16x8(uintx4 x) {
+  uintx4 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float lo = __builtin_bit_cast(float, x[i] << 16);
+    const float hi = __builtin_bit_cast(float, x[i] & 0xffff0000u);
+    half2v h = {(_Float16)lo, (_Float16)hi};
+    r[i] = __builtin_bit_cast(unsigned int, h);
+  }
+  return r;
+}
+
+// 16-byte chunk swizzles of the LDS tiles (rows of D halfs = D/8 chunks).
+//  K tile: operand reads take one chunk of 32 consecutive rows -> spread the chunk index over rows.
+//  V tile: transpose reads take 64 contiguous bytes of 4 consecutive rows -> move rows to
+//          different 64-byte parts of the 256-byte bank period.
+template <int D> __device__ __forceinline__ int k_swz(int row) { return D == 64 ? ((row >> 1) & 7) : (row & 15); }
+template <int D> __device__ __forceinline__ int v_swz(int row) { return D == 64 ? (((row >> 1) & 1) << 2) : ((row & 3) << 2); }
+
+typedef unsigned char __attribute__((address_space(3)))* lds_ptr_t;
+typedef const int32_t __attribute__((address_space(4)))* cint_ptr_t;
+
+// Asynchronous global -> LDS copy of one 64 x D tile: D/8 instructions, each moving 16 bytes
+// per lane; the data of lane l lands at lds + j*1024 + l*16.  `off` holds the per-lane
+// source byte offsets from `tile` (a wave-uniform base).  The copies are issued from
+// inline assembly so that the compiler's own wait-count insertion does not serialise
+// them; completion is awaited explicitly with wait_vm<N>() (vector memory operations
+// retire in order, so "at most N outstanding" means everything older than the N youngest
+// has landed).
+template <int D>
+__device__ __forceinline__ void tile_load_async(const unsigned short* tile, const unsigned (&off)[D / 8],
+                                                unsigned lds_addr) {
+#pragma unroll
+  for (int j = 0; j < D / 8; ++j)
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_addr + j * 1024), "v"(off[j]), "s"(tile) : "memory", "m0");
+}
+
+
+template <int N> __device__ __forceinline__ void wait_vm() {
+  asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
+}
+
+__device__ __forceinline__ void lds_wait() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
+// 4 consecutive output values of one row: fp32, or packed fp16/bf16
+template <bool BF16>
+__device__ __forceinline__ void store_out4(void* obase, int64_t elem_off, bool out_f32, float x0, float x1,
+                                           float x2, float x3) {
+  if (out_f32) {
+    const floatx4 w = {x0, x1, x2, x3};
+    *reinterpret_cast<floatx4*>((float*)obase + elem_off) = w;
+  } else {
+    uintx2 w;
+    if constexpr (BF16) {
+      typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+      const bf2 a = {(__bf16)x0, (__bf16)x1}, c = {(__bf16)x2, (__bf16)x3};
+      w[0] = __builtin_bit_cast(unsigned int, a); w[1] = __builtin_bit_cast(unsigned int, c);
+    } else {
+      const half2v a = {(_Float16)x0, (_Float16)x1}, c = {(_Float16)x2, (_Float16)x3};
+      w[0] = __builtin_bit_cast(unsigned int, a); w[1] = __builtin_bit_cast(unsigned int, c);
+    }
+    *reinterpret_cast<uintx2*>((unsigned short*)obase + elem_off) = w;
+  }
+}
+
+
+// Swizzle for tiles that are read both ways (operand reads of 32 consecutive rows and
+// transpose reads of 4 consecutive rows x 64 bytes): a bijection of the row bits that
+// separates both access patterns over the 64 LDS banks.
+template <int D> __device__ __forceinline__ int u_swz(int row) {
+  if (D == 64) { const int x = (row >> 1) & 7; return ((x & 1) << 2) | (x >> 1); }
+  return ((row & 3) << 2) | ((row >> 2) & 3);
+}
+
+}  // namespace bsattn

@@ -1,0 +1,89 @@
+"""GPU parity of the backward kernels against the CPU oracle's closed-form gradients
+(algebra of fa2_bwd.py, pinned on the CPU against torch.autograd through the naive fp32 path).
+Tolerances as the forward: max-abs 2e-2 (fp16) / 3e-2 (bf16); rel-L2 1e-3 on fp32-typed outputs
+(bf16-typed outputs are limited by the output cast itself, 1.7e-3)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import bsattn_oracle as orc
+from helpers import make_qkv, uniform_block_mask, causal_block_mask, errors, f32
+
+pytestmark = pytest.mark.gpu
+MAXABS = {torch.float16: 2e-2, torch.bfloat16: 3e-2}
+
+
+def run_case(dev, B, H, N, D, dtype, mask, seed, out_fp32):
+    import fa2_custom_mask as fm
+    q, k, v, do = make_qkv(B, H, N, D, dtype, seed, n=4)
+    sc = 1.0 / np.sqrt(D)
+    dq_r, dk_r, dv_r, _ = orc.attention_backward(f32(q), f32(k), f32(v), mask.numpy(), sc, f32(do))
+    o_r, lse_r = orc.naive_attention(f32(q), f32(k), f32(v), mask.numpy(), sc, return_lse=True)
+    o, lse, dq, dk, dv = fm.attention_forward_backward(q.to(dev), k.to(dev), v.to(dev), mask.to(dev), sc,
+                                                       do.to(dev), out_fp32=out_fp32)
+    torch.cuda.synchronize()
+    want = torch.float32 if out_fp32 else dtype
+    for name, got, ref in (("O", o, o_r), ("dQ", dq, dq_r), ("dK", dk, dk_r), ("dV", dv, dv_r)):
+        assert got.dtype == want and tuple(got.shape) == (B, H, N, D)
+        ma, rl = errors(got, ref)
+        print("%s B%d H%d N%d D%d %s fp32out=%s: max-abs %.3e rel-L2 %.3e" % (name, B, H, N, D, dtype, out_fp32, ma, rl))
+        assert ma <= MAXABS[dtype]
+        assert rl <= (1e-3 if (dtype == torch.float16 or out_fp32) else 3e-3)
+    fin = np.isfinite(lse_r)
+    assert np.abs(lse.cpu().numpy()[fin] - lse_r[fin]).max() <= 2e-3
+    return dq, dk, dv
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [64, 128])
+def test_small(dev, D, dtype):
+    run_case(dev, 2, 2, 512, D, dtype, uniform_block_mask(2, 2, 8, 0.4, 3), 11, True)
+    run_case(dev, 2, 2, 512, D, dtype, uniform_block_mask(2, 2, 8, 0.4, 3), 11, False)
+
+
+def test_shared_causal_mask_c5_shape_small(dev):
+    """C5's structure at reduced size: mask shared across heads, block-causal keep 0.25, bf16 D=128."""
+    run_case(dev, 2, 4, 1024, 128, torch.bfloat16, causal_block_mask(1, 1, 16, 0.25, 5), 1238, True)
+
+
+def test_empty_rows_and_columns(dev):
+    m = uniform_block_mask(1, 2, 8, 0.3, 2)
+    m[0, 0, 3, :] = False          # a query block without keys: dQ = 0 there
+    m[0, 1, :, 5] = False          # a key block nobody attends to: dK = dV = 0 there
+    dq, dk, dv = run_case(dev, 1, 2, 512, 64, torch.float16, m, 8, True)
+    assert float(dq[0, 0, 192:256].abs().max()) == 0.0
+    assert float(dk[0, 1, 320:384].abs().max()) == 0.0 and float(dv[0, 1, 320:384].abs().max()) == 0.0
+
+
+def test_autograd_path(dev):
+    """o.backward(do) through flash_attention_custom_mask, as the reference's users call it."""
+    import fa2_custom_mask as fm
+    B, H, N, D = 1, 2, 512, 64
+    q, k, v, do = make_qkv(B, H, N, D, torch.float16, 21, n=4)
+    mask = uniform_block_mask(1, 1, 8, 0.5, 21)
+    sc = 0.125
+    qd, kd, vd = [x.to(dev).requires_grad_(True) for x in (q, k, v)]
+    o = fm.flash_attention_custom_mask(qd, kd, vd, mask.to(dev), sc)
+    o.backward(do.to(dev))
+    dq_r, dk_r, dv_r, _ = orc.attention_backward(f32(q), f32(k), f32(v), mask.numpy(), sc, f32(do))
+    for got, ref in ((qd.grad, dq_r), (kd.grad, dk_r), (vd.grad, dv_r)):
+        assert got.dtype == torch.float16
+        ma, rl = errors(got, ref)
+        assert ma <= 2e-2 and rl <= 1e-3
+    # all-false mask: zeros forward (fa2_custom_mask.py:49-51) and zero gradients
+    qd.grad = None
+    z = fm.flash_attention_custom_mask(qd, kd, vd, torch.zeros(1, 1, 8, 8, dtype=torch.bool, device=dev), sc)
+    z.backward(do.to(dev))
+    assert float(z.abs().max()) == 0.0 and float(qd.grad.abs().max()) == 0.0
+
+
+def test_invariant_rowsum_ds_zero(dev):
+    """With dO = O-independent constant along d and v = const, dS rows sum to zero, so dQ = dK = 0."""
+    import fa2_custom_mask as fm
+    B, H, N, D = 1, 1, 1024, 64
+    q, k, v, do = make_qkv(B, H, N, D, torch.float16, 4, n=4)
+    mask = uniform_block_mask(1, 1, 16, 0.3, 4)
+    vc = torch.ones_like(v) * 0.5
+    _, _, dq, dk, dv = fm.attention_forward_backward(q.to(dev), k.to(dev), vc.to(dev), mask.to(dev), 0.125,
+                                                     do.to(dev), out_fp32=True)
+    assert float(dq.abs().max()) <= 2e-3 and float(dk.abs().max()) <= 2e-3
