@@ -46,6 +46,11 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only-keep", type=float, default=None,
+                    help="profiling aid: run only forward passes at this kept-tile ratio and exit")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="profiling aid: run a plain 256 MiB device copy a few times and exit "
+                         "(reference reading for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (heads / row blocks shard without "
@@ -55,11 +60,18 @@ def main():
     import numpy as np
     import torch
     import fa2_custom_mask as fm
-    from fa2_custom_mask import fa2_custom_mask as host
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     dev = torch.device("cuda:0")
+    if args.copy_calibration:
+        src = torch.ones(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes": 256 << 20, "copies": 5}))
+        return
     g = torch.Generator().manual_seed(SEED)
     q, k, v = [torch.randn(1, 1, N, D, generator=g).to(torch.float16) for _ in range(3)]
     masks = {}
@@ -72,8 +84,18 @@ def main():
     lists = {r: fm.block_mask_to_lists(masks[r].to(dev)) for r in KEEPS}
     kept = {r: int(lists[r].counts[1]) for r in KEEPS}
 
+    plans = {r: fm.ForwardPlan(qd, kd, vd, lists[r], sm_scale) for r in KEEPS}
+
     def fwd(r):
-        return host._forward(qd, kd, vd, lists[r], sm_scale, torch.float16, True)
+        return plans[r].run()
+
+    if args.only_keep is not None:
+        for _ in range(args.warmup + args.steps):
+            fwd(args.only_keep)
+        torch.cuda.synchronize()
+        print(json.dumps({"only_keep": args.only_keep, "kept_tiles": kept[args.only_keep],
+                          "launches": args.warmup + args.steps}))
+        return
 
     # ---- headline: K timed steps at keep 1.0 ----
     for _ in range(args.warmup):
@@ -128,21 +150,26 @@ def main():
         "parity_max_abs_vs_oracle": parity,
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": None,
-                     "kernel": "fwd_kernel<64,false> + combine_kernel<64,false> (one bsattn_fwd call)"},
+                     "kernel": "fwd_kernel<64,false> + combine_kernel<64,false> (one bsattn_fwd call)",
+                     "algorithmic_flops_per_launch": tile_flops(kept[1.0])},
     }
     if not args.no_cpu:
-        # CPU baseline: the oracle's C port of the naive path, all host threads, on the first
-        # 4096 query rows of the same keep-1.0 workload (every key), reported in the metric's unit.
-        rows = 4096
+        # CPU baseline: the oracle's C port of the naive path on all host threads, the whole
+        # keep-1.0 workload (every query row, every key), median of 3 passes after a short warm-up,
+        # reported in the metric's unit.
         qf, kf, vf = q.float().numpy(), k.float().numpy(), v.float().numpy()
-        c_oracle.naive_fwd(qf, kf, vf, masks[1.0].numpy(), sm_scale, 0, 64)
-        t0 = time.perf_counter()
-        c_oracle.naive_fwd(qf, kf, vf, masks[1.0].numpy(), sm_scale, 0, rows)
-        dt = time.perf_counter() - t0
-        out["cpu_baseline"] = {"value": round(4.0 * rows * N * D / dt / 1e12, 5), "unit": "TFLOP/s",
+        c_oracle.naive_fwd(qf, kf, vf, masks[1.0].numpy(), sm_scale, 0, 256)
+        dts = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            c_oracle.naive_fwd(qf, kf, vf, masks[1.0].numpy(), sm_scale, 0, N)
+            dts.append(time.perf_counter() - t0)
+        dt = sorted(dts)[1]
+        out["cpu_baseline"] = {"value": round(4.0 * N * N * D / dt / 1e12, 5), "unit": "TFLOP/s",
                                "cores": c_oracle.num_threads(), "kind": "port",
-                               "sample": "first %d of %d query rows, all keys, keep 1.0, fp32 naive "
-                                         "masked softmax (oracle C port, OpenMP), %.2f s" % (rows, N, dt)}
+                               "sample": "whole workload (%d query rows x %d keys, keep 1.0), fp32 naive masked "
+                                         "softmax, oracle C port with OpenMP, median of 3 passes, %.2f s per pass"
+                                         % (N, N, dt)}
     print(json.dumps(out))
 
 

@@ -71,6 +71,33 @@ def _forward(q, k, v, lists, sm_scale, out_dtype, want_lse):
     return o, lse
 
 
+class ForwardPlan:
+    """A forward call with every buffer allocated and every C argument marshalled once; run()
+    only enqueues the kernels.  For loops that repeat the same shapes (serving, benchmarks)."""
+
+    def __init__(self, q, k, v, lists, sm_scale, out_dtype=None, stream=None):
+        B, H, N, D = q.shape
+        self.q, self.k, self.v, self.lists = _prep(q), _prep(k), _prep(v), lists
+        out_dtype = out_dtype or q.dtype
+        self.o = torch.empty((B, H, N, D), dtype=out_dtype, device=q.device)
+        self.lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device)
+        wsb = _ext.fwd_workspace(B, H, N, D)
+        self.ws = torch.empty(wsb, dtype=torch.uint8, device=q.device)
+        self._keep = (_ext.strides4(self.q), _ext.strides4(self.k), _ext.strides4(self.v), _ext.strides4(self.o))
+        stream = stream if stream is not None else torch.cuda.current_stream(q.device)
+        self._args = (self.q.data_ptr(), self.k.data_ptr(), self.v.data_ptr(), self.o.data_ptr(),
+                      self.lse.data_ptr(), lists.row_ptr.data_ptr(), lists.col_idx.data_ptr(), lists.Bm,
+                      lists.Hm, B, H, N, D, _ext.dtype_code(q.dtype), _ext.dtype_code(out_dtype),
+                      float(sm_scale)) + self._keep + (self.ws.data_ptr(), wsb, ctypes.c_void_p(stream.cuda_stream))
+        self._fn = _ext.lib().bsattn_fwd
+
+    def run(self):
+        rc = self._fn(*self._args)
+        if rc != 0:
+            _ext.check(rc, "bsattn_fwd")
+        return self.o, self.lse
+
+
 def _backward(q, k, v, o, do, lse, lists, lists_t, sm_scale, out_dtype):
     B, H, N, D = q.shape
     q, k, v, o, do = _prep(q), _prep(k), _prep(v), _prep(o), _prep(do)
