@@ -100,23 +100,20 @@ __device__ __forceinline__ void recentre(floatx16& s0, floatx16& s1, floatx16 (&
 
 // Number of wavefronts of a workgroup: 2 per SIMD at D=64 (256 VGPRs each), 1 per SIMD at D=128.
 template <int D> struct FwdCfg {
+#ifdef EXP_NW
+  static constexpr int NW = EXP_NW;
+#else
   static constexpr int NW = D == 64 ? 8 : 4;
+#endif
   static constexpr int TILE_BYTES = 64 * 2 * D;             // one K or V tile in LDS
   static constexpr int WAVE_LDS = 2 * TILE_BYTES;           // K buffer + V buffer
-  static constexpr int ML_BYTES = NW * 2 * 64 * 4;          // exchange of (m, l) per query
-  static constexpr int LDS_BYTES = NW * WAVE_LDS + ML_BYTES;
+  static constexpr int ML_BYTES = NW * 2 * 64 * 4 + 64;     // exchange of (m, l) per query + the tile counter
+  static constexpr int COLS_CAP = 2048;                     // column indices of the range kept in LDS
+  static constexpr int LDS_BYTES = NW * WAVE_LDS + ML_BYTES + COLS_CAP * 4;
   static constexpr int R = TILE_BYTES / 256;                // accumulator registers exchanged per round
   static constexpr int ROUNDS = D / R;
   static constexpr int QPW = (R / 4) / NW;                  // output quads per wavefront and round
 };
-
-// share of wavefront w in a segment of n tiles starting at a
-__device__ __forceinline__ int share_begin(int a, int n, int w, int NW) {
-#ifdef EXP_WEIGHTED
-  if (NW == 8) { const int cum = w <= 4 ? 3 * w : 12 + 2 * (w - 4); return a + (cum * n) / 20; }
-#endif
-  return a + (w * n) / NW;
-}
 
 template <int D, bool BF16>
 __global__ __launch_bounds__(FwdCfg<D>::NW * 64)
@@ -159,14 +156,35 @@ void fwd_kernel(const FwdParams prm) {
   const unsigned short* vg = (const unsigned short*)prm.v + b * prm.vs[0] + h * prm.vs[1];
   const float qk_scale = prm.qk_scale;
 
-  // per-lane source byte offsets of the asynchronous tile loads (loop invariant)
-  unsigned koff[CPR], voff[CPR];
+  // Per-lane source byte offsets of the asynchronous tile loads (loop invariant).  Copy
+  // instruction j covers rows [64j/CPR, 64(j+1)/CPR) of the tile; the row part of the offset is
+  // added to the (scalar) tile pointer, the per-lane part only depends on j through the chunk
+  // swizzle, whose pattern repeats with period KPER in j (K) or not at all (V).
+  constexpr int RPI = 64 / CPR;                 // tile rows per copy instruction
+  constexpr int KPER = D == 64 ? 2 : 4;         // period of the K swizzle in copy instructions
+  unsigned koff[KPER], voff[1];
+  {
+    const int row0 = lane / CPR, ch = lane % CPR;
 #pragma unroll
-  for (int j = 0; j < CPR; ++j) {
-    const int c = j * 64 + lane, row = c / CPR, ch = c % CPR;
-    koff[j] = 2u * (unsigned)(row * (int)prm.ks[2] + ((ch ^ k_swz<D>(row)) * 8));
-    voff[j] = 2u * (unsigned)(row * (int)prm.vs[2] + ((ch ^ v_swz<D>(row)) * 8));
+    for (int par = 0; par < KPER; ++par)
+      koff[par] = 2u * (unsigned)(row0 * (int)prm.ks[2] + ((ch ^ k_swz<D>(par * RPI + row0)) * 8));
+    voff[0] = 2u * (unsigned)(row0 * (int)prm.vs[2] + ((ch ^ v_swz<D>(row0)) * 8));
   }
+  static_assert(D == 64 || D == 128, "swizzle periods below are derived for 64 and 128");
+  auto k_copy = [&](const unsigned short* tile, int j) {
+    tile_load_async_one(tile + (int64_t)j * RPI * prm.ks[2], koff[j % KPER], lds_k_addr + j * 1024);
+  };
+  auto v_copy = [&](const unsigned short* tile, int j) {
+    tile_load_async_one(tile + (int64_t)j * RPI * prm.vs[2], voff[0], lds_v_addr + j * 1024);
+  };
+  auto k_copy_all = [&](const unsigned short* tile) {
+#pragma unroll
+    for (int j = 0; j < CPR; ++j) k_copy(tile, j);
+  };
+  auto v_copy_all = [&](const unsigned short* tile) {
+#pragma unroll
+    for (int j = 0; j < CPR; ++j) v_copy(tile, j);
+  };
   // per-lane LDS byte offsets of the operand reads.  K fragment (kb, s): row 32kb+ln, chunk 2s+g
   int kaddr[2][KS];
 #pragma unroll
@@ -193,29 +211,39 @@ void fwd_kernel(const FwdParams prm) {
   Ta = __builtin_amdgcn_s_memrealtime();
 #endif
   const uintx4 ones_frag = {g == 0 ? 0x3c003c00u : 0u, 0u, 0u, 0u};
-  // Asynchronous copies of one wavefront are issued in the order K(j), V(j), K(j'), V(j'), ...
-  // (j' the wavefront's next tile): K(j') as soon as the first product of tile j has consumed
-  // the K buffer, V(j') as soon as the second product has consumed the V buffer, so every wait
-  // below allows exactly the one younger copy (CPR instructions) in flight.  `pre` is the tile
-  // whose K copy has been issued ahead (-1: none); its V copy is held back across the merge of
-  // a row block, which borrows the V buffers.
-  int pre = -1;
+  // Tiles of the range are handed out to the wavefronts dynamically (an LDS counter), because
+  // the two wavefronts of a SIMD do not progress at the same rate: each wavefront owns a current
+  // tile `cur` and has already drawn its next one `nxt`, so that it can prefetch it.  Tiles are
+  // drawn in list order, so a wavefront's tiles increase, and `cur >= seg_b` means "nothing left
+  // for me in this row block".
+  // Asynchronous copies of one wavefront are issued in the order K(cur), V(cur), K(nxt), V(nxt),
+  // ...: K(nxt) as soon as the first product of tile cur has consumed the K buffer, V(nxt) as soon
+  // as the second product has consumed the V buffer, so every wait below allows exactly the one
+  // younger copy (CPR instructions) in flight.  kdone / vdone name the tile whose copy into this
+  // wavefront's K / V buffer has been issued; a V copy is held back across the merge of a row
+  // block, which borrows the V buffers.
+#ifdef EXP_TIMING
+  long long tk[8] = {0,0,0,0,0,0,0,0}; int ntile = 0;
+#endif
+  int* ctr = reinterpret_cast<int*>(ml + NW * 2 * 64);
+  // The column indices of the range are staged in LDS: a scalar load per tile would put its
+  // whole latency in front of the tile's first LDS wait (scalar loads return out of order, so
+  // any wait on the shared counter becomes a wait for all of them).
+  int* lcols = ctr + 16;
+  for (int i = threadIdx.x; i < g1 - g0 && i < C::COLS_CAP; i += NW * 64) lcols[i] = prm.col_idx[g0 + i];
+  if (threadIdx.x == 0) *ctr = g0 + 2 * NW;
+  __syncthreads();
+  auto col_of = [&](int tile) { return tile - g0 < C::COLS_CAP ? lcols[tile - g0] : (int)cols[tile]; };
+  int cur = g0 + w, nxt = g0 + NW + w;      // the first two rounds are fixed
+  int cb_nxt = nxt < g1 ? __builtin_amdgcn_readfirstlane(col_of(nxt)) : 0;   // column block of tile nxt
+  int kdone = -1, vdone = -1;
   bool first_seg = true;
   int t = g0;
   while (t < g1) {
     const int row_s = rp[r], row_e = rp[r + 1];
     if (row_e <= t) { ++r; continue; }          // row block without kept tiles in the range
-    const int seg_a = t, seg_b = row_e < g1 ? row_e : g1, n = seg_b - seg_a;
-    const int ma = share_begin(seg_a, n, w, NW), mb = share_begin(seg_a, n, w + 1, NW);
-    // this wavefront's first tile in the next segment of the range (-1: none or not adjacent)
-    int nxt_seg = -1;
-    if (seg_b < g1) {
-      int r2 = r + 1;
-      while (rp[r2 + 1] <= seg_b) ++r2;
-      const int e2 = rp[r2 + 1] < g1 ? rp[r2 + 1] : g1, n2 = e2 - seg_b;
-      const int a2 = share_begin(seg_b, n2, w, NW), b2 = share_begin(seg_b, n2, w + 1, NW);
-      if (a2 < b2) nxt_seg = a2;
-    }
+    const int seg_a = t, seg_b = row_e < g1 ? row_e : g1;
+    const bool mine = cur < seg_b;      // this wavefront processes at least one tile of the row block
 
     floatx16 oacc[DB][2];
     float m_i[2] = {0.f, 0.f}, l_i[2] = {0.f, 0.f};
@@ -226,12 +254,10 @@ void fwd_kernel(const FwdParams prm) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) oacc[db][qb][i] = 0.f;
 
-    if (ma < mb) {
-      if (pre != ma) {   // nothing issued ahead for this tile
-        const int cb = cols[ma];
-        tile_load_async<D>(kg + (int64_t)cb * 64 * prm.ks[2], koff, lds_k_addr);
-      }
-      tile_load_async<D>(vg + (int64_t)cols[ma] * 64 * prm.vs[2], voff, lds_v_addr);
+    if (mine) {
+      const int cbc = __builtin_amdgcn_readfirstlane(col_of(cur));
+      if (kdone != cur) { k_copy_all(kg + (int64_t)cbc * 64 * prm.ks[2]); kdone = cur; }
+      if (vdone != cur) { v_copy_all(vg + (int64_t)cbc * 64 * prm.vs[2]); vdone = cur; }
       // ---- Q fragments (second operand of S^T = K Q^T): lane owns query ln (+32 qb) ----
       uintx4 qf[2][KS];
 #pragma unroll
@@ -266,71 +292,43 @@ void fwd_kernel(const FwdParams prm) {
       if (nseg == 0) Tq = __builtin_amdgcn_s_memrealtime();
 #endif
 
-      for (int j = ma; j < mb; ++j) {
-        const int nxt = j + 1 < mb ? j + 1 : nxt_seg;
-        const bool has1 = nxt >= 0;
-        const int cbn = has1 ? cols[nxt] : 0;
+      while (cur < seg_b) {
+#ifdef EXP_TIMING
+        long long c0 = __builtin_readcyclecounter(), c1;
+#endif
+        // draw the tile after next; the value is only needed at the end of this tile
+        int drawn = 0;
+        if (lane == 0) drawn = atomicAdd(ctr, 1);
+        const bool has1 = nxt < g1;
+        const int cbn = cb_nxt;
 
-        // ---- S^T[kb][qb] = K[kb] Q[qb]^T (- m_i when FOLD) ----
-        // K fragments are read one step ahead of the MFMAs that consume them.
-        wait_vm<CPR>();  // K(j) has landed (V(j), issued after it, may still be in flight)
-        floatx16 sacc[2][2];
+        // The tile is processed as four blocks so that the matrix cores and the vector ALU of
+        // this wavefront overlap: [1] scores of query block 0, [2] scores of query block 1
+        // interleaved with the softmax numerators of block 0, [3] second product of block 0
+        // interleaved with the numerators of block 1, [4] second product of block 1.
+        // operand fragments of the tile are read from LDS once, all at once (the read latency is a
+        // multiple of an MFMA's issue interval), and serve both query blocks
+        uintx4 kfr[2][KS], vfr[4][DB];
+        auto scores = [&](int qb, floatx16& s0, floatx16& s1) {   // S^T[.][qb] = K Q[qb]^T (- m_i when FOLD)
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) sacc[kb][qb][i] = 0.f;
-        {
-          uintx4 ka[2], kn[2];
-#pragma unroll
-          for (int kb = 0; kb < 2; ++kb) ka[kb] = *reinterpret_cast<const uintx4*>(lds_k + kaddr[kb][0]);
+          for (int i = 0; i < 16; ++i) { s0[i] = 0.f; s1[i] = 0.f; }
 #pragma unroll
           for (int s = 0; s < KS; ++s) {
-            if (s + 1 < KS) {
-#pragma unroll
-              for (int kb = 0; kb < 2; ++kb) kn[kb] = *reinterpret_cast<const uintx4*>(lds_k + kaddr[kb][s + 1]);
-            }
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-              for (int qb = 0; qb < 2; ++qb) sacc[kb][qb] = mfma_qk<BF16>(ka[kb], qf[qb][s], sacc[kb][qb]);
-            __builtin_amdgcn_sched_barrier(0);
-            if (s + 1 < KS) { ka[0] = kn[0]; ka[1] = kn[1]; }
+            s0 = mfma_qk<BF16>(kfr[0][s], qf[qb][s], s0);
+            s1 = mfma_qk<BF16>(kfr[1][s], qf[qb][s], s1);
           }
           if constexpr (FOLD) {
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-              for (int qb = 0; qb < 2; ++qb) sacc[kb][qb] = mfma_qk<BF16>(ones_frag, mfrag[qb], sacc[kb][qb]);
+            s0 = mfma_qk<BF16>(ones_frag, mfrag[qb], s0);
+            s1 = mfma_qk<BF16>(ones_frag, mfrag[qb], s1);
           }
-        }
-        // every K fragment has been read: refill the K buffer with the wavefront's next tile
-        if (has1) tile_load_async<D>(kg + (int64_t)cbn * 64 * prm.ks[2], koff, lds_k_addr);
-
-        // ---- softmax numerators, one query per lane ----
-        // Fast path: P = exp2(score - m_i) with the reference m_i left alone; the row sum of the
-        // fp16-rounded P (what the second product consumes) is accumulated with dot2.  If a
-        // lane's sum grows by 2^14 or more (or is not finite), some P left the safe fp16 range:
-        // recentre() moves m_i to the tile's row maximum and the tile's numerators are redone.
+        };
         uintx4 pf[4][2];  // P^T operand fragments: [16-key slice][qb]
+        auto read_v = [&]() {
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb) {
-          float lnew = softmax_tile<FOLD>(sacc[0][qb], sacc[1][qb], qk_scale, m_i[qb], l_i[qb], pf, qb);
-          if (__any(fresh || !(lnew - l_i[qb] < 16384.0f))) {
-            recentre<DB, FOLD>(sacc[0][qb], sacc[1][qb], oacc, qb, qk_scale, m_i[qb], l_i[qb], mfrag[qb], fresh, g);
-            lnew = softmax_tile<FOLD>(sacc[0][qb], sacc[1][qb], qk_scale, m_i[qb], l_i[qb], pf, qb);
-          }
-          l_i[qb] = lnew;
-        }
-        fresh = false;
-
-        // ---- O^T[db][qb] += V^T[db] P^T[qb]; V^T fragments by LDS transpose reads, one step ahead ----
-        if (has1) wait_vm<CPR>(); else wait_vm<0>();  // V(j) has landed (K(nxt) may be in flight)
-        {
-          auto read_v = [&](int ts, uintx4 (&dst)[DB]) {
+          for (int ts = 0; ts < 4; ++ts)
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
+              uintx4 a;
 #pragma unroll
               for (int jh = 0; jh < 2; ++jh) {
                 const int key = 16 * ts + 8 * jh + vkey0, col = 32 * db + vcol0;
@@ -338,41 +336,114 @@ void fwd_kernel(const FwdParams prm) {
                 const short4v rr = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                     (short4v __attribute__((address_space(3)))*)(lds_v + addr));
                 const uintx2 r2 = __builtin_bit_cast(uintx2, rr);
-                dst[db][2 * jh] = r2[0]; dst[db][2 * jh + 1] = r2[1];
+                a[2 * jh] = r2[0]; a[2 * jh + 1] = r2[1];
               }
+              if constexpr (BF16) a = bf16x8_to_f16x8(a);
+              vfr[ts][db] = a;
             }
-          };
-          uintx4 va[DB], vn[DB];
-          read_v(0, va);
+        };
+        auto second = [&](int qb) {        // O^T[.][qb] += V^T P^T[qb]
 #pragma unroll
-          for (int ts = 0; ts < 4; ++ts) {
-            if (ts + 1 < 4) read_v(ts + 1, vn);
+          for (int ts = 0; ts < 4; ++ts)
 #pragma unroll
-            for (int db = 0; db < DB; ++db) {
-              uintx4 af = va[db];
-              if constexpr (BF16) af = bf16x8_to_f16x8(af);
-#pragma unroll
-              for (int qb = 0; qb < 2; ++qb)
-                oacc[db][qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, af),
-                                                                     __builtin_bit_cast(half8, pf[ts][qb]),
-                                                                     oacc[db][qb], 0, 0, 0);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            if (ts + 1 < 4) {
-#pragma unroll
-              for (int db = 0; db < DB; ++db) va[db] = vn[db];
-            }
+            for (int db = 0; db < DB; ++db)
+              oacc[db][qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, vfr[ts][db]),
+                                                                   __builtin_bit_cast(half8, pf[ts][qb]),
+                                                                   oacc[db][qb], 0, 0, 0);
+        };
+        // Softmax numerators, one query per lane.  Fast path: P = exp2(score - m_i) with the
+        // reference m_i left alone; the row sum of the fp16-rounded P (what the second product
+        // consumes) is accumulated with dot2.  If a lane's sum grows by 2^14 or more (or is not
+        // finite), some P left the safe fp16 range: recentre() moves m_i to the tile's row maximum
+        // and the numerators are redone from the scores, which are still live.
+        auto settle = [&](int qb, floatx16& s0, floatx16& s1, float lnew) {
+          if (__any(fresh || !(lnew - l_i[qb] < 16384.0f))) {
+            recentre<DB, FOLD>(s0, s1, oacc, qb, qk_scale, m_i[qb], l_i[qb], mfrag[qb], fresh, g);
+            lnew = softmax_tile<FOLD>(s0, s1, qk_scale, m_i[qb], l_i[qb], pf, qb);
           }
+          l_i[qb] = lnew;
+        };
+
+        floatx16 sa0, sa1, sb0, sb1;
+#ifdef EXP_TIMING
+#define TICK(k) { c1 = __builtin_readcyclecounter(); tk[k] += c1 - c0; c0 = c1; }
+#else
+#define TICK(k)
+#endif
+        wait_vm<CPR>();  // K(j) has landed (V(j), issued after it, may still be in flight)
+        TICK(0)
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int s = 0; s < KS; ++s) kfr[kb][s] = *reinterpret_cast<const uintx4*>(lds_k + kaddr[kb][s]);
+        lds_wait();   // the K fragments (and the drawn tile number) have arrived: the K buffer is free
+        const int nn = __builtin_amdgcn_readfirstlane(drawn);
+        const int cb_nn_v = nn < g1 ? col_of(nn) : 0;     // looked up now, needed at the end of the tile
+        // the next K tile can be copied in now
+        if (has1) { k_copy_all(kg + (int64_t)cbn * 64 * prm.ks[2]); kdone = nxt; }
+        // [1]
+        scores(0, sa0, sa1);
+        __builtin_amdgcn_sched_barrier(0);
+#ifdef EXP_TIMING
+        asm volatile("" :: "v"(sa1[15]));
+#endif
+        TICK(1)
+        // [2]
+        scores(1, sb0, sb1);
+        float lnew0 = softmax_tile<FOLD>(sa0, sa1, qk_scale, m_i[0], l_i[0], pf, 0);
+#pragma unroll
+        for (int it = 0; it < 2 * KS + (FOLD ? 2 : 0); ++it) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x002, 64 / (2 * KS + (FOLD ? 2 : 0)) + 1, 0);   // its share of the VALU work
         }
-        // refill the V buffer, except across the merge below, which borrows it
-        if (has1 && j + 1 < mb) tile_load_async<D>(vg + (int64_t)cbn * 64 * prm.vs[2], voff, lds_v_addr);
+        __builtin_amdgcn_sched_barrier(0);
+#ifdef EXP_TIMING
+        asm volatile("" :: "v"(sb1[15]), "v"(lnew0));
+#endif
+        TICK(2)
+        settle(0, sa0, sa1, lnew0);
+        TICK(3)
+        if (has1) wait_vm<CPR>(); else wait_vm<0>();  // V(cur) has landed (K(nxt) may be in flight)
+        TICK(4)
+        read_v();
+        lds_wait();   // the V fragments sit in registers: the next V tile can be copied in, except
+        // across the merge below, which borrows the V buffer
+        if (nxt < seg_b) { v_copy_all(vg + (int64_t)cbn * 64 * prm.vs[2]); vdone = nxt; }
+        // [3]
+        second(0);
+        float lnew1 = softmax_tile<FOLD>(sb0, sb1, qk_scale, m_i[1], l_i[1], pf, 1);
+#pragma unroll
+        for (int it = 0; it < 4 * DB; ++it) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, 64 / (4 * DB) + 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#ifdef EXP_TIMING
+        asm volatile("" :: "v"(oacc[DB-1][0][15]), "v"(lnew1));
+#endif
+        TICK(5)
+        settle(1, sb0, sb1, lnew1);
+        TICK(6)
+        fresh = false;
+        // [4]
+        second(1);
+        __builtin_amdgcn_sched_barrier(0);
+#ifdef EXP_TIMING
+        asm volatile("" :: "v"(oacc[DB-1][1][15]));
+#endif
+        TICK(7)
+#ifdef EXP_TIMING
+        ++ntile;
+#endif
+        cur = nxt;
+        nxt = nn;
+        cb_nxt = __builtin_amdgcn_readfirstlane(cb_nn_v);
+#ifdef EXP_TIMING
+        { c1 = __builtin_readcyclecounter(); tk[7] += c1 - c0; }
+#endif
       }  // tiles of this wavefront
-      pre = nxt_seg;
     }
 
-#ifdef EXP_TIMING
-    if (nseg == 0) Tb = __builtin_amdgcn_s_memrealtime();
-#endif
     // ---- merge the wavefronts' results of this row block through LDS ----
     // Each wavefront publishes (m, l) per query and, round by round, R accumulator registers in
     // its own V buffer ([register][lane] floats); in every round each wavefront reduces QPW
@@ -385,8 +456,8 @@ void fwd_kernel(const FwdParams prm) {
       if (g == 0) {
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
-          ml[(w * 2 + 0) * 64 + qb * 32 + ln] = ma < mb ? m_i[qb] : -INFINITY;
-          ml[(w * 2 + 1) * 64 + qb * 32 + ln] = ma < mb ? lsum[qb] : 0.f;
+          ml[(w * 2 + 0) * 64 + qb * 32 + ln] = mine ? m_i[qb] : -INFINITY;
+          ml[(w * 2 + 1) * 64 + qb * 32 + ln] = mine ? lsum[qb] : 0.f;
         }
       }
       const bool full = (seg_a == row_s) && (seg_b == row_e);
@@ -396,12 +467,12 @@ void fwd_kernel(const FwdParams prm) {
       void* obase = out_base(prm, b, h);
 #pragma unroll
       for (int rd = 0; rd < C::ROUNDS; ++rd) {
-        if (ma < mb) {
-          float* mine = reinterpret_cast<float*>(lds_v);
+        if (mine) {
+          float* own = reinterpret_cast<float*>(lds_v);
 #pragma unroll
           for (int e = 0; e < C::R; ++e) {
             const int idx = rd * C::R + e;
-            mine[e * 64 + lane] = oacc[idx / 32][(idx / 16) & 1][idx & 15];
+            own[e * 64 + lane] = oacc[idx / 32][(idx / 16) & 1][idx & 15];
           }
         }
         __syncthreads();
@@ -430,7 +501,7 @@ void fwd_kernel(const FwdParams prm) {
           float x[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int pw = 0; pw < NW; ++pw) {
-            if (share_begin(seg_a, n, pw, NW) < share_begin(seg_a, n, pw + 1, NW)) {   // wavefront pw contributed
+            if (ml[(pw * 2 + 0) * 64] != -INFINITY) {   // wavefront pw contributed to this row block
               const float* src = reinterpret_cast<const float*>(lds + pw * C::WAVE_LDS + C::TILE_BYTES);
 #pragma unroll
               for (int e = 0; e < 4; ++e) x[e] += wgt[pw][qb] * src[(4 * quad + e) * 64 + lane];
@@ -473,7 +544,8 @@ void fwd_kernel(const FwdParams prm) {
 #ifdef EXP_TIMING
   Td = __builtin_amdgcn_s_memrealtime();
   if ((wg % 61) == 5 && lane == 0 && (w == 0 || w == 7))
-    printf("wg=%d w=%d tiles=%d segs=%d | setup %lld | Q+first loads %lld | seg0 tiles %lld | seg0 merge %lld | rest %lld | total %lld (x10ns)\n", wg, w, g1 - g0, nseg, Ta - T0, Tq - Ta, Tb - Tq, Tc - Tb, Td - Tc, Td - T0);
+    printf("wg=%d w=%d mytiles=%d per tile: waitK %lld [1] %lld [2] %lld settle0 %lld waitV+dma %lld [3] %lld settle1 %lld [4] %lld\n", wg, w, ntile, tk[0]/ntile, tk[1]/ntile, tk[2]/ntile, tk[3]/ntile, tk[4]/ntile, tk[5]/ntile, tk[6]/ntile, tk[7]/ntile);
+  if ((wg % 61) == 5 && lane == 0 && (w == 0 || w == 7)) printf("wg=%d w=%d tiles=%d segs=%d | setup %lld | Q+first loads %lld | seg0 tiles %lld | seg0 merge %lld | rest %lld | total %lld (x10ns)\n", wg, w, g1 - g0, nseg, Ta - T0, Tq - Ta, Tb - Tq, Tc - Tb, Td - Tc, Td - T0);
 #endif
 }
 

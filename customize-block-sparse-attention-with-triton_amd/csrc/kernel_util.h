@@ -79,12 +79,22 @@ typedef const int32_t __attribute__((address_space(4)))* cint_ptr_t;
 template <int D>
 __device__ __forceinline__ void tile_load_async(const unsigned short* tile, const unsigned (&off)[D / 8],
                                                 unsigned lds_addr) {
+#ifdef EXP_LOADSTEP
+#pragma unroll
+  for (int j = 0; j < D / 8; j += EXP_LOADSTEP)
+#else
 #pragma unroll
   for (int j = 0; j < D / 8; ++j)
+#endif
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :: "s"(lds_addr + j * 1024), "v"(off[j]), "s"(tile) : "memory", "m0");
 }
 
+
+// one instruction of tile_load_async: 64 x 16 bytes to lds_addr (+ lane*16)
+__device__ __forceinline__ void tile_load_async_one(const unsigned short* tile, unsigned off, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(lds_addr), "v"(off), "s"(tile) : "memory", "m0");
+}
 
 template <int N> __device__ __forceinline__ void wait_vm() {
   asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
