@@ -100,11 +100,7 @@ __device__ __forceinline__ void recentre(floatx16& s0, floatx16& s1, floatx16 (&
 
 // Number of wavefronts of a workgroup: 2 per SIMD at D=64 (256 VGPRs each), 1 per SIMD at D=128.
 template <int D> struct FwdCfg {
-#ifdef EXP_NW
-  static constexpr int NW = EXP_NW;
-#else
   static constexpr int NW = D == 64 ? 8 : 4;
-#endif
   static constexpr int TILE_BYTES = 64 * 2 * D;             // one K or V tile in LDS
   static constexpr int WAVE_LDS = 2 * TILE_BYTES;           // K buffer + V buffer
   static constexpr int ML_BYTES = NW * 2 * 64 * 4 + 64;     // exchange of (m, l) per query + the tile counter
@@ -115,7 +111,7 @@ template <int D> struct FwdCfg {
   static constexpr int QPW = (R / 4) / NW;                  // output quads per wavefront and round
 };
 
-template <int D, bool BF16>
+template <int D, bool BF16, bool ROWS>
 __global__ __launch_bounds__(FwdCfg<D>::NW * 64)
 void fwd_kernel(const FwdParams prm) {
   using C = FwdCfg<D>;
@@ -127,9 +123,6 @@ void fwd_kernel(const FwdParams prm) {
   constexpr int ROWB = 2 * D;      // bytes per LDS row
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
 
-#ifdef EXP_TIMING
-  const long long T0 = __builtin_amdgcn_s_memrealtime(); long long Ta = 0, Tb = 0, Tc = 0, Td = 0, Tq = 0; int nseg = 0;
-#endif
   const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int ln = lane & 31, g = lane >> 5;
@@ -141,9 +134,10 @@ void fwd_kernel(const FwdParams prm) {
   const cint_ptr_t rp = (cint_ptr_t)(uintptr_t)(prm.row_ptr + (int64_t)mh * nb);
   const cint_ptr_t cols = (cint_ptr_t)(uintptr_t)prm.col_idx;
   const HeadSplit hs = head_split(rp, nb, prm.W, NW);
-  if (wg >= hs.Peff) return;
-  const int g0 = split_begin(hs, wg), g1 = split_begin(hs, wg + 1);
-  if (g0 >= g1) return;
+  // a head without kept tiles: the row-per-wavefront driver still has to write its zeros
+  if (wg >= (ROWS && hs.T == 0 ? 1 : hs.Peff)) return;
+  const int g0 = hs.T > 0 ? split_begin(hs, wg) : hs.lo, g1 = hs.T > 0 ? split_begin(hs, wg + 1) : hs.lo;
+  if (!ROWS && g0 >= g1) return;
 
   unsigned char* lds_k = lds + w * C::WAVE_LDS;
   unsigned char* lds_v = lds_k + C::TILE_BYTES;
@@ -199,354 +193,403 @@ void fwd_kernel(const FwdParams prm) {
   const int vblk = lane >> 4, vs_ = lane & 15;
   const int vkey0 = 4 * (vblk >> 1) + (vs_ >> 2), vcol0 = 16 * (vblk & 1) + 4 * (vs_ & 3);
 
-  // first row block of the range: largest r with rp[r] <= g0 < rp[r+1]
-  int r;
-  {
-    int lo = 0, hi = nb;  // invariant: rp[lo] <= g0 < rp[hi]
-    while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (rp[mid] <= g0) lo = mid; else hi = mid; }
-    r = lo;
-  }
-
-#ifdef EXP_TIMING
-  Ta = __builtin_amdgcn_s_memrealtime();
-#endif
   const uintx4 ones_frag = {g == 0 ? 0x3c003c00u : 0u, 0u, 0u, 0u};
-  // Tiles of the range are handed out to the wavefronts dynamically (an LDS counter), because
-  // the two wavefronts of a SIMD do not progress at the same rate: each wavefront owns a current
-  // tile `cur` and has already drawn its next one `nxt`, so that it can prefetch it.  Tiles are
-  // drawn in list order, so a wavefront's tiles increase, and `cur >= seg_b` means "nothing left
-  // for me in this row block".
-  // Asynchronous copies of one wavefront are issued in the order K(cur), V(cur), K(nxt), V(nxt),
-  // ...: K(nxt) as soon as the first product of tile cur has consumed the K buffer, V(nxt) as soon
-  // as the second product has consumed the V buffer, so every wait below allows exactly the one
-  // younger copy (CPR instructions) in flight.  kdone / vdone name the tile whose copy into this
-  // wavefront's K / V buffer has been issued; a V copy is held back across the merge of a row
-  // block, which borrows the V buffers.
-#ifdef EXP_TIMING
-  long long tk[8] = {0,0,0,0,0,0,0,0}; int ntile = 0;
-#endif
-  int* ctr = reinterpret_cast<int*>(ml + NW * 2 * 64);
-  // The column indices of the range are staged in LDS: a scalar load per tile would put its
-  // whole latency in front of the tile's first LDS wait (scalar loads return out of order, so
-  // any wait on the shared counter becomes a wait for all of them).
-  int* lcols = ctr + 16;
-  for (int i = threadIdx.x; i < g1 - g0 && i < C::COLS_CAP; i += NW * 64) lcols[i] = prm.col_idx[g0 + i];
-  if (threadIdx.x == 0) *ctr = g0 + 2 * NW;
-  __syncthreads();
-  auto col_of = [&](int tile) { return tile - g0 < C::COLS_CAP ? lcols[tile - g0] : (int)cols[tile]; };
-  int cur = g0 + w, nxt = g0 + NW + w;      // the first two rounds are fixed
-  int cb_nxt = nxt < g1 ? __builtin_amdgcn_readfirstlane(col_of(nxt)) : 0;   // column block of tile nxt
-  int kdone = -1, vdone = -1;
-  bool first_seg = true;
-  int t = g0;
-  while (t < g1) {
-    const int row_s = rp[r], row_e = rp[r + 1];
-    if (row_e <= t) { ++r; continue; }          // row block without kept tiles in the range
-    const int seg_a = t, seg_b = row_e < g1 ? row_e : g1;
-    const bool mine = cur < seg_b;      // this wavefront processes at least one tile of the row block
 
-    floatx16 oacc[DB][2];
-    float m_i[2] = {0.f, 0.f}, l_i[2] = {0.f, 0.f};
+  // ---- state of the row block a wavefront is working on, and the steps both drivers share ----
+  uintx4 qf[2][KS];          // Q fragments (second operand of S^T = K Q^T): lane owns query ln (+32 qb)
+  floatx16 oacc[DB][2];
+  // m_i: reference exponent of the row (exp2 domain), l_i: per-lane partial sum of P (this lane's
+  // half of the keys), both relative to m_i.  m_i starts at 0 and is re-centred on the first tile
+  // and whenever a tile produces a P above 2^14.
+  float m_i[2], l_i[2];
+  // FOLD: "-m_i" enters the scores through one extra contraction slice, ones x (-m_hi, -m_lo)
+  uintx4 mfrag[2];
+  bool fresh = true;
+
+  auto reset_acc = [&]() {
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) oacc[db][qb][i] = 0.f;
-
-    if (mine) {
-      const int cbc = __builtin_amdgcn_readfirstlane(col_of(cur));
-      if (kdone != cur) { k_copy_all(kg + (int64_t)cbc * 64 * prm.ks[2]); kdone = cur; }
-      if (vdone != cur) { v_copy_all(vg + (int64_t)cbc * 64 * prm.vs[2]); vdone = cur; }
-      // ---- Q fragments (second operand of S^T = K Q^T): lane owns query ln (+32 qb) ----
-      uintx4 qf[2][KS];
 #pragma unroll
-      for (int qb = 0; qb < 2; ++qb) {
-        const unsigned short* qrow = qg + (int64_t)(r * 64 + qb * 32 + ln) * prm.qs[2];
+    for (int qb = 0; qb < 2; ++qb) { m_i[qb] = 0.f; l_i[qb] = 0.f; mfrag[qb] = uintx4{0u, 0u, 0u, 0u}; }
+    fresh = true;
+  };
+  auto load_q = [&](int r) {
 #pragma unroll
-        for (int s = 0; s < KS; ++s) qf[qb][s] = *reinterpret_cast<const uintx4*>(qrow + 16 * s + 8 * g);
-      }
-      // vmcnt(0), visible to the compiler: Q is complete here, so that no vector-memory waits
-      // of its own end up inside the tile loop (they would also wait for the tile prefetches)
-      __builtin_amdgcn_s_waitcnt(0x0F70);
-      if constexpr (FOLD) {
-        // fold sm_scale*log2(e) into Q once per row block: the scores leave the MFMA already in
-        // the exp2 domain (fp16 rounding of the scaled Q perturbs an exponent by ~1e-4)
+    for (int qb = 0; qb < 2; ++qb) {
+      const unsigned short* qrow = qg + (int64_t)(r * 64 + qb * 32 + ln) * prm.qs[2];
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-          for (int s = 0; s < KS; ++s) {
-            const uintx4 raw = qf[qb][s];
-            const uintx4 scaled = {scale_half2(raw[0], qk_scale), scale_half2(raw[1], qk_scale),
-                                   scale_half2(raw[2], qk_scale), scale_half2(raw[3], qk_scale)};
-            qf[qb][s] = scaled;
-          }
-      }
-      // m_i: reference exponent of the row (exp2 domain), l_i: per-lane partial sum of P (this
-      // lane's half of the keys), both relative to m_i.  m_i starts at 0 and is re-centred on
-      // the first tile and whenever a tile produces a P above 2^14.
-      // FOLD: "-m_i" enters the scores through one extra contraction slice, ones x (-m_hi, -m_lo)
-      uintx4 mfrag[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
-      bool fresh = true;
-#ifdef EXP_TIMING
-      if (nseg == 0) Tq = __builtin_amdgcn_s_memrealtime();
-#endif
-
-      while (cur < seg_b) {
-#ifdef EXP_TIMING
-        long long c0 = __builtin_readcyclecounter(), c1;
-#endif
-        // draw the tile after next; the value is only needed at the end of this tile
-        int drawn = 0;
-        if (lane == 0) drawn = atomicAdd(ctr, 1);
-        const bool has1 = nxt < g1;
-        const int cbn = cb_nxt;
-
-        // The tile is processed as four blocks so that the matrix cores and the vector ALU of
-        // this wavefront overlap: [1] scores of query block 0, [2] scores of query block 1
-        // interleaved with the softmax numerators of block 0, [3] second product of block 0
-        // interleaved with the numerators of block 1, [4] second product of block 1.
-        // operand fragments of the tile are read from LDS once, all at once (the read latency is a
-        // multiple of an MFMA's issue interval), and serve both query blocks
-        uintx4 kfr[2][KS], vfr[4][DB];
-        auto scores = [&](int qb, floatx16& s0, floatx16& s1) {   // S^T[.][qb] = K Q[qb]^T (- m_i when FOLD)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) { s0[i] = 0.f; s1[i] = 0.f; }
-#pragma unroll
-          for (int s = 0; s < KS; ++s) {
-            s0 = mfma_qk<BF16>(kfr[0][s], qf[qb][s], s0);
-            s1 = mfma_qk<BF16>(kfr[1][s], qf[qb][s], s1);
-          }
-          if constexpr (FOLD) {
-            s0 = mfma_qk<BF16>(ones_frag, mfrag[qb], s0);
-            s1 = mfma_qk<BF16>(ones_frag, mfrag[qb], s1);
-          }
-        };
-        uintx4 pf[4][2];  // P^T operand fragments: [16-key slice][qb]
-        auto read_v = [&]() {
-#pragma unroll
-          for (int ts = 0; ts < 4; ++ts)
-#pragma unroll
-            for (int db = 0; db < DB; ++db) {
-              uintx4 a;
-#pragma unroll
-              for (int jh = 0; jh < 2; ++jh) {
-                const int key = 16 * ts + 8 * jh + vkey0, col = 32 * db + vcol0;
-                const int addr = key * ROWB + (((col >> 3) ^ v_swz<D>(key)) * 16) + (col & 7) * 2;
-                const short4v rr = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (short4v __attribute__((address_space(3)))*)(lds_v + addr));
-                const uintx2 r2 = __builtin_bit_cast(uintx2, rr);
-                a[2 * jh] = r2[0]; a[2 * jh + 1] = r2[1];
-              }
-              if constexpr (BF16) a = bf16x8_to_f16x8(a);
-              vfr[ts][db] = a;
-            }
-        };
-        auto second = [&](int qb) {        // O^T[.][qb] += V^T P^T[qb]
-#pragma unroll
-          for (int ts = 0; ts < 4; ++ts)
-#pragma unroll
-            for (int db = 0; db < DB; ++db)
-              oacc[db][qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, vfr[ts][db]),
-                                                                   __builtin_bit_cast(half8, pf[ts][qb]),
-                                                                   oacc[db][qb], 0, 0, 0);
-        };
-        // Softmax numerators, one query per lane.  Fast path: P = exp2(score - m_i) with the
-        // reference m_i left alone; the row sum of the fp16-rounded P (what the second product
-        // consumes) is accumulated with dot2.  If a lane's sum grows by 2^14 or more (or is not
-        // finite), some P left the safe fp16 range: recentre() moves m_i to the tile's row maximum
-        // and the numerators are redone from the scores, which are still live.
-        auto settle = [&](int qb, floatx16& s0, floatx16& s1, float lnew) {
-          if (__any(fresh || !(lnew - l_i[qb] < 16384.0f))) {
-            recentre<DB, FOLD>(s0, s1, oacc, qb, qk_scale, m_i[qb], l_i[qb], mfrag[qb], fresh, g);
-            lnew = softmax_tile<FOLD>(s0, s1, qk_scale, m_i[qb], l_i[qb], pf, qb);
-          }
-          l_i[qb] = lnew;
-        };
-
-        floatx16 sa0, sa1, sb0, sb1;
-#ifdef EXP_TIMING
-#define TICK(k) { c1 = __builtin_readcyclecounter(); tk[k] += c1 - c0; c0 = c1; }
-#else
-#define TICK(k)
-#endif
-        wait_vm<CPR>();  // K(j) has landed (V(j), issued after it, may still be in flight)
-        TICK(0)
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int s = 0; s < KS; ++s) kfr[kb][s] = *reinterpret_cast<const uintx4*>(lds_k + kaddr[kb][s]);
-        lds_wait();   // the K fragments (and the drawn tile number) have arrived: the K buffer is free
-        const int nn = __builtin_amdgcn_readfirstlane(drawn);
-        const int cb_nn_v = nn < g1 ? col_of(nn) : 0;     // looked up now, needed at the end of the tile
-        // the next K tile can be copied in now
-        if (has1) { k_copy_all(kg + (int64_t)cbn * 64 * prm.ks[2]); kdone = nxt; }
-        // [1]
-        scores(0, sa0, sa1);
-        __builtin_amdgcn_sched_barrier(0);
-#ifdef EXP_TIMING
-        asm volatile("" :: "v"(sa1[15]));
-#endif
-        TICK(1)
-        // [2]
-        scores(1, sb0, sb1);
-        float lnew0 = softmax_tile<FOLD>(sa0, sa1, qk_scale, m_i[0], l_i[0], pf, 0);
-#pragma unroll
-        for (int it = 0; it < 2 * KS + (FOLD ? 2 : 0); ++it) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
-          __builtin_amdgcn_sched_group_barrier(0x002, 64 / (2 * KS + (FOLD ? 2 : 0)) + 1, 0);   // its share of the VALU work
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#ifdef EXP_TIMING
-        asm volatile("" :: "v"(sb1[15]), "v"(lnew0));
-#endif
-        TICK(2)
-        settle(0, sa0, sa1, lnew0);
-        TICK(3)
-        if (has1) wait_vm<CPR>(); else wait_vm<0>();  // V(cur) has landed (K(nxt) may be in flight)
-        TICK(4)
-        read_v();
-        lds_wait();   // the V fragments sit in registers: the next V tile can be copied in, except
-        // across the merge below, which borrows the V buffer
-        if (nxt < seg_b) { v_copy_all(vg + (int64_t)cbn * 64 * prm.vs[2]); vdone = nxt; }
-        // [3]
-        second(0);
-        float lnew1 = softmax_tile<FOLD>(sb0, sb1, qk_scale, m_i[1], l_i[1], pf, 1);
-#pragma unroll
-        for (int it = 0; it < 4 * DB; ++it) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x002, 64 / (4 * DB) + 1, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#ifdef EXP_TIMING
-        asm volatile("" :: "v"(oacc[DB-1][0][15]), "v"(lnew1));
-#endif
-        TICK(5)
-        settle(1, sb0, sb1, lnew1);
-        TICK(6)
-        fresh = false;
-        // [4]
-        second(1);
-        __builtin_amdgcn_sched_barrier(0);
-#ifdef EXP_TIMING
-        asm volatile("" :: "v"(oacc[DB-1][1][15]));
-#endif
-        TICK(7)
-#ifdef EXP_TIMING
-        ++ntile;
-#endif
-        cur = nxt;
-        nxt = nn;
-        cb_nxt = __builtin_amdgcn_readfirstlane(cb_nn_v);
-#ifdef EXP_TIMING
-        { c1 = __builtin_readcyclecounter(); tk[7] += c1 - c0; }
-#endif
-      }  // tiles of this wavefront
+      for (int s = 0; s < KS; ++s) qf[qb][s] = *reinterpret_cast<const uintx4*>(qrow + 16 * s + 8 * g);
     }
-
-    // ---- merge the wavefronts' results of this row block through LDS ----
-    // Each wavefront publishes (m, l) per query and, round by round, R accumulator registers in
-    // its own V buffer ([register][lane] floats); in every round each wavefront reduces QPW
-    // groups of 4 registers (4 consecutive head-dimension values of one query per lane) over all
-    // contributing wavefronts and writes them out.
-    {
-      float lsum[2];
+    // vmcnt(0), visible to the compiler: Q is complete here, so that no vector-memory waits of
+    // its own end up inside the tile loop (they would also wait for the tile prefetches)
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    if constexpr (FOLD) {
+      // fold sm_scale*log2(e) into Q once per row block: the scores leave the MFMA already in
+      // the exp2 domain (fp16 rounding of the scaled Q perturbs an exponent by ~1e-4)
 #pragma unroll
-      for (int qb = 0; qb < 2; ++qb) lsum[qb] = l_i[qb] + __shfl_xor(l_i[qb], 32);
-      if (g == 0) {
+      for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+          const uintx4 raw = qf[qb][s];
+          const uintx4 scaled = {scale_half2(raw[0], qk_scale), scale_half2(raw[1], qk_scale),
+                                 scale_half2(raw[2], qk_scale), scale_half2(raw[3], qk_scale)};
+          qf[qb][s] = scaled;
+        }
+    }
+  };
+
+  // One 64 x 64 tile whose K and V copies have been issued (K first).  has1: the wavefront has a
+  // next tile, in column block cbn, whose K copy is issued as soon as this tile's K fragments sit
+  // in registers; copy_v: its V copy may be issued too, as soon as this tile's V fragments sit in
+  // registers.  Copies are therefore issued in the order K(cur), V(cur), K(nxt), V(nxt), ..., and
+  // every wait allows exactly the one younger copy (CPR instructions) in flight.  `mid` runs once
+  // the first LDS wait of the tile has passed (the place to pick up earlier LDS results).
+  // The tile is processed as four blocks so that the matrix cores and the vector ALU of this
+  // wavefront overlap: [1] scores of query block 0, [2] scores of query block 1 interleaved with
+  // the softmax numerators of block 0, [3] second product of block 0 interleaved with the
+  // numerators of block 1, [4] second product of block 1.  Operand fragments are read from LDS
+  // once, all at once (the read latency is a multiple of an MFMA's issue interval), and serve
+  // both query blocks.
+  auto tile = [&](bool has1, int cbn, bool copy_v, auto&& mid) {
+    uintx4 kfr[2][KS], vfr[4][DB];
+    uintx4 pf[4][2];  // P^T operand fragments: [16-key slice][qb]
+    auto scores = [&](int qb, floatx16& s0, floatx16& s1) {   // S^T[.][qb] = K Q[qb]^T (- m_i when FOLD)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) { s0[i] = 0.f; s1[i] = 0.f; }
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        s0 = mfma_qk<BF16>(kfr[0][s], qf[qb][s], s0);
+        s1 = mfma_qk<BF16>(kfr[1][s], qf[qb][s], s1);
+      }
+      if constexpr (FOLD) {
+        s0 = mfma_qk<BF16>(ones_frag, mfrag[qb], s0);
+        s1 = mfma_qk<BF16>(ones_frag, mfrag[qb], s1);
+      }
+    };
+    auto read_v = [&]() {
+#pragma unroll
+      for (int ts = 0; ts < 4; ++ts)
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          uintx4 a;
+#pragma unroll
+          for (int jh = 0; jh < 2; ++jh) {
+            const int key = 16 * ts + 8 * jh + vkey0, col = 32 * db + vcol0;
+            const int addr = key * ROWB + (((col >> 3) ^ v_swz<D>(key)) * 16) + (col & 7) * 2;
+            const short4v rr = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (short4v __attribute__((address_space(3)))*)(lds_v + addr));
+            const uintx2 r2 = __builtin_bit_cast(uintx2, rr);
+            a[2 * jh] = r2[0]; a[2 * jh + 1] = r2[1];
+          }
+          if constexpr (BF16) a = bf16x8_to_f16x8(a);
+          vfr[ts][db] = a;
+        }
+    };
+    auto second = [&](int qb) {        // O^T[.][qb] += V^T P^T[qb]
+#pragma unroll
+      for (int ts = 0; ts < 4; ++ts)
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+          oacc[db][qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, vfr[ts][db]),
+                                                               __builtin_bit_cast(half8, pf[ts][qb]),
+                                                               oacc[db][qb], 0, 0, 0);
+    };
+    // Softmax numerators, one query per lane.  Fast path: P = exp2(score - m_i) with the
+    // reference m_i left alone; the row sum of the fp16-rounded P (what the second product
+    // consumes) is accumulated with dot2.  If a lane's sum grows by 2^14 or more (or is not
+    // finite), some P left the safe fp16 range: recentre() moves m_i to the tile's row maximum
+    // and the numerators are redone from the scores, which are still live.
+    auto settle = [&](int qb, floatx16& s0, floatx16& s1, float lnew) {
+      if (__any(fresh || !(lnew - l_i[qb] < 16384.0f))) {
+        recentre<DB, FOLD>(s0, s1, oacc, qb, qk_scale, m_i[qb], l_i[qb], mfrag[qb], fresh, g);
+        lnew = softmax_tile<FOLD>(s0, s1, qk_scale, m_i[qb], l_i[qb], pf, qb);
+      }
+      l_i[qb] = lnew;
+    };
+
+    floatx16 sa0, sa1, sb0, sb1;
+    wait_vm<CPR>();  // K(cur) has landed (V(cur), issued after it, may still be in flight)
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int s = 0; s < KS; ++s) kfr[kb][s] = *reinterpret_cast<const uintx4*>(lds_k + kaddr[kb][s]);
+    lds_wait();      // the K fragments have arrived: the K buffer is free
+    mid();
+    if (has1) k_copy_all(kg + (int64_t)cbn * 64 * prm.ks[2]);
+    // [1]
+    scores(0, sa0, sa1);
+    __builtin_amdgcn_sched_barrier(0);
+    // [2]
+    scores(1, sb0, sb1);
+    float lnew0 = softmax_tile<FOLD>(sa0, sa1, qk_scale, m_i[0], l_i[0], pf, 0);
+#pragma unroll
+    for (int it = 0; it < 2 * KS + (FOLD ? 2 : 0); ++it) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+      __builtin_amdgcn_sched_group_barrier(0x002, 64 / (2 * KS + (FOLD ? 2 : 0)) + 1, 0);   // its share of the VALU work
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    settle(0, sa0, sa1, lnew0);
+    if (has1) wait_vm<CPR>(); else wait_vm<0>();  // V(cur) has landed (K(nxt) may be in flight)
+    read_v();
+    lds_wait();      // the V fragments have arrived: the V buffer is free
+    if (copy_v) v_copy_all(vg + (int64_t)cbn * 64 * prm.vs[2]);
+    // [3]
+    second(0);
+    float lnew1 = softmax_tile<FOLD>(sb0, sb1, qk_scale, m_i[1], l_i[1], pf, 1);
+#pragma unroll
+    for (int it = 0; it < 4 * DB; ++it) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 64 / (4 * DB) + 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    settle(1, sb0, sb1, lnew1);
+    fresh = false;
+    // [4]
+    second(1);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  int* ctr = reinterpret_cast<int*>(ml + NW * 2 * 64);
+  int* lcols = ctr + 16;
+  // The column indices of the range are staged in LDS: a scalar load per tile would put its whole
+  // latency in front of the tile's first LDS wait (scalar loads return out of order, so any wait
+  // on the shared counter becomes a wait for all of them).
+  auto stage_cols = [&](int t_lo, int t_hi) {
+    for (int i = threadIdx.x; i < t_hi - t_lo && i < C::COLS_CAP; i += NW * 64) lcols[i] = prm.col_idx[t_lo + i];
+  };
+
+  if constexpr (ROWS) {
+    // ================= one wavefront per row block =================
+    // The workgroup owns the row blocks whose first kept tile lies in its range [g0, g1); they are
+    // handed out to the wavefronts through the LDS counter, and a wavefront runs a whole row block
+    // alone and writes its result directly: no merge, no partials.
+    int r_lo, r_hi;
+    {
+      int lo = -1, hi = nb;   // smallest r with rp[r] >= g0
+      while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (rp[mid] >= g0) hi = mid; else lo = mid; }
+      r_lo = hi;
+      lo = -1; hi = nb;       // smallest r with rp[r] >= g1
+      while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (rp[mid] >= g1) hi = mid; else lo = mid; }
+      r_hi = hi;
+      if (wg >= hs.Peff - 1) r_hi = nb;    // trailing row blocks without kept tiles
+      if (wg == 0) r_lo = 0;               // leading ones
+    }
+    const int t_lo = rp[r_lo];
+    stage_cols(t_lo, rp[r_hi]);
+    if (threadIdx.x == 0) *ctr = r_lo + 2 * NW;
+    __syncthreads();
+    auto col_of = [&](int t) { return t - t_lo < C::COLS_CAP ? lcols[t - t_lo] : (int)cols[t]; };
+    void* obase = out_base(prm, b, h);
+    int row = r_lo + w, row_next = r_lo + NW + w;     // the first two rounds are fixed
+    int kdone = -1;                                    // tile whose K and V copies were issued ahead
+    while (row < r_hi) {
+      int drawn = 0;
+      if (lane == 0) drawn = atomicAdd(ctr, 1);       // the row block after next
+      const int ta = rp[row], tb = rp[row + 1];
+      // first tile of the next row block of this wavefront (prefetched under the last tile)
+      const int tn = row_next < r_hi ? rp[row_next] : 0;
+      const bool next_has = row_next < r_hi && rp[row_next + 1] > tn;
+      if (ta < tb) {
+        if (kdone != ta) {
+          const int cb = __builtin_amdgcn_readfirstlane(col_of(ta));
+          k_copy_all(kg + (int64_t)cb * 64 * prm.ks[2]);
+          v_copy_all(vg + (int64_t)cb * 64 * prm.vs[2]);
+        }
+        reset_acc();
+        load_q(row);
+        for (int j = ta; j < tb; ++j) {
+          const bool last = j + 1 == tb;
+          const bool has1 = !last || next_has;
+          const int cbn = has1 ? __builtin_amdgcn_readfirstlane(col_of(last ? tn : j + 1)) : 0;
+          tile(has1, cbn, has1, [] {});
+        }
+        kdone = next_has ? tn : -1;
+        // normalise and write the row block
+        float lsum[2];
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb) lsum[qb] = l_i[qb] + __shfl_xor(l_i[qb], 32);
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
-          ml[(w * 2 + 0) * 64 + qb * 32 + ln] = mine ? m_i[qb] : -INFINITY;
-          ml[(w * 2 + 1) * 64 + qb * 32 + ln] = mine ? lsum[qb] : 0.f;
+          const float inv = 1.0f / lsum[qb];
+          const int64_t qrow = (int64_t)(row * 64 + qb * 32 + ln);
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4)
+              store_out4<BF16>(obase, qrow * prm.os[2] + 32 * db + 8 * i4 + 4 * g, prm.out_f32,
+                               oacc[db][qb][4 * i4] * inv, oacc[db][qb][4 * i4 + 1] * inv,
+                               oacc[db][qb][4 * i4 + 2] * inv, oacc[db][qb][4 * i4 + 3] * inv);
+          if (prm.lse != nullptr && g == 0)
+            prm.lse[((int64_t)bh * prm.N) + qrow] = (m_i[qb] + __builtin_amdgcn_logf(lsum[qb])) * 0.6931471805599453f;
+        }
+      } else {
+        // row block without kept tiles: O = 0, lse = -inf
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb) {
+          const int64_t qrow = (int64_t)(row * 64 + qb * 32 + ln);
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4)
+              store_out4<BF16>(obase, qrow * prm.os[2] + 32 * db + 8 * i4 + 4 * g, prm.out_f32, 0.f, 0.f, 0.f, 0.f);
+          if (prm.lse != nullptr && g == 0) prm.lse[((int64_t)bh * prm.N) + qrow] = -INFINITY;
         }
       }
-      const bool full = (seg_a == row_s) && (seg_b == row_e);
-      float wgt[NW][2];   // weight of wavefront p's partial for this lane's query of block qb
-      float M[2], L[2];
-      float* slot = prm.ws + ((((int64_t)bh * prm.W + wg) * 2) + (first_seg ? 0 : 1)) * partial_floats(D);
-      void* obase = out_base(prm, b, h);
+      row = row_next;
+      row_next = __builtin_amdgcn_readfirstlane(drawn);
+    }
+  } else {
+    // ================= all wavefronts on one row block at a time =================
+    // Tiles of the range are handed out to the wavefronts dynamically (the LDS counter), because
+    // the two wavefronts of a SIMD do not progress at the same rate: each wavefront owns a current
+    // tile `cur` and has already drawn its next one `nxt`, so that it can prefetch it.  Tiles are
+    // drawn in list order, so a wavefront's tiles increase, and `cur >= seg_b` means "nothing left
+    // for me in this row block".  kdone / vdone name the tile whose copy into this wavefront's
+    // K / V buffer has been issued; a V copy is held back across the merge of a row block, which
+    // borrows the V buffers.
+    // first row block of the range: largest r with rp[r] <= g0 < rp[r+1]
+    int r;
+    {
+      int lo = 0, hi = nb;  // invariant: rp[lo] <= g0 < rp[hi]
+      while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (rp[mid] <= g0) lo = mid; else hi = mid; }
+      r = lo;
+    }
+    stage_cols(g0, g1);
+    if (threadIdx.x == 0) *ctr = g0 + 2 * NW;
+    __syncthreads();
+    auto col_of = [&](int t) { return t - g0 < C::COLS_CAP ? lcols[t - g0] : (int)cols[t]; };
+    int cur = g0 + w, nxt = g0 + NW + w;      // the first two rounds are fixed
+    int cb_nxt = nxt < g1 ? __builtin_amdgcn_readfirstlane(col_of(nxt)) : 0;   // column block of tile nxt
+    int kdone = -1, vdone = -1;
+    bool first_seg = true;
+    int t = g0;
+    while (t < g1) {
+      const int row_s = rp[r], row_e = rp[r + 1];
+      if (row_e <= t) { ++r; continue; }          // row block without kept tiles in the range
+      const int seg_a = t, seg_b = row_e < g1 ? row_e : g1;
+      const bool mine = cur < seg_b;      // this wavefront processes at least one tile of the row block
+      reset_acc();
+      if (mine) {
+        const int cbc = __builtin_amdgcn_readfirstlane(col_of(cur));
+        if (kdone != cur) { k_copy_all(kg + (int64_t)cbc * 64 * prm.ks[2]); kdone = cur; }
+        if (vdone != cur) { v_copy_all(vg + (int64_t)cbc * 64 * prm.vs[2]); vdone = cur; }
+        load_q(r);
+        while (cur < seg_b) {
+          // draw the tile after next; the value is picked up inside the tile
+          int drawn = 0;
+          if (lane == 0) drawn = atomicAdd(ctr, 1);
+          const bool has1 = nxt < g1, copy_v = nxt < seg_b;
+          int nn = 0, cb_nn_v = 0;
+          tile(has1, cb_nxt, copy_v, [&] {
+            nn = __builtin_amdgcn_readfirstlane(drawn);
+            cb_nn_v = nn < g1 ? col_of(nn) : 0;     // looked up now, needed at the end of the tile
+          });
+          if (has1) kdone = nxt;
+          if (copy_v) vdone = nxt;
+          cur = nxt;
+          nxt = nn;
+          cb_nxt = __builtin_amdgcn_readfirstlane(cb_nn_v);
+        }  // tiles of this wavefront
+      }
+
+      // ---- merge the wavefronts' results of this row block through LDS ----
+      // Each wavefront publishes (m, l) per query and, round by round, R accumulator registers in
+      // its own V buffer ([register][lane] floats); in every round each wavefront reduces QPW
+      // groups of 4 registers (4 consecutive head-dimension values of one query per lane) over all
+      // contributing wavefronts and writes them out.
+      {
+        float lsum[2];
 #pragma unroll
-      for (int rd = 0; rd < C::ROUNDS; ++rd) {
-        if (mine) {
-          float* own = reinterpret_cast<float*>(lds_v);
-#pragma unroll
-          for (int e = 0; e < C::R; ++e) {
-            const int idx = rd * C::R + e;
-            own[e * 64 + lane] = oacc[idx / 32][(idx / 16) & 1][idx & 15];
-          }
-        }
-        __syncthreads();
-        if (rd == 0) {
+        for (int qb = 0; qb < 2; ++qb) lsum[qb] = l_i[qb] + __shfl_xor(l_i[qb], 32);
+        if (g == 0) {
 #pragma unroll
           for (int qb = 0; qb < 2; ++qb) {
-            float mm = -INFINITY;
+            ml[(w * 2 + 0) * 64 + qb * 32 + ln] = mine ? m_i[qb] : -INFINITY;
+            ml[(w * 2 + 1) * 64 + qb * 32 + ln] = mine ? lsum[qb] : 0.f;
+          }
+        }
+        const bool full = (seg_a == row_s) && (seg_b == row_e);
+        float wgt[NW][2];   // weight of wavefront p's partial for this lane's query of block qb
+        float M[2], L[2];
+        float* slot = prm.ws + ((((int64_t)bh * prm.W + wg) * 2) + (first_seg ? 0 : 1)) * partial_floats(D);
+        void* obase = out_base(prm, b, h);
 #pragma unroll
-            for (int pw = 0; pw < NW; ++pw) mm = fmaxf(mm, ml[(pw * 2 + 0) * 64 + qb * 32 + ln]);
-            float ll = 0.f;
+        for (int rd = 0; rd < C::ROUNDS; ++rd) {
+          if (mine) {
+            float* own = reinterpret_cast<float*>(lds_v);
+#pragma unroll
+            for (int e = 0; e < C::R; ++e) {
+              const int idx = rd * C::R + e;
+              own[e * 64 + lane] = oacc[idx / 32][(idx / 16) & 1][idx & 15];
+            }
+          }
+          __syncthreads();
+          if (rd == 0) {
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb) {
+              float mm = -INFINITY;
+#pragma unroll
+              for (int pw = 0; pw < NW; ++pw) mm = fmaxf(mm, ml[(pw * 2 + 0) * 64 + qb * 32 + ln]);
+              float ll = 0.f;
+#pragma unroll
+              for (int pw = 0; pw < NW; ++pw) {
+                const float mp = ml[(pw * 2 + 0) * 64 + qb * 32 + ln];
+                const float wp = mp == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mp - mm);
+                wgt[pw][qb] = wp;
+                ll += wp * ml[(pw * 2 + 1) * 64 + qb * 32 + ln];
+              }
+              M[qb] = mm; L[qb] = ll;
+            }
+          }
+#pragma unroll
+          for (int tq = 0; tq < C::QPW; ++tq) {
+            const int quad = w * C::QPW + tq;              // group of 4 registers within this round
+            const int idx0 = rd * C::R + 4 * quad;         // accumulator register index (db, qb, i16)
+            const int db = idx0 / 32, qb = (idx0 / 16) & 1, i4 = (idx0 & 15) / 4;
+            float x[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int pw = 0; pw < NW; ++pw) {
-              const float mp = ml[(pw * 2 + 0) * 64 + qb * 32 + ln];
-              const float wp = mp == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mp - mm);
-              wgt[pw][qb] = wp;
-              ll += wp * ml[(pw * 2 + 1) * 64 + qb * 32 + ln];
+              if (ml[(pw * 2 + 0) * 64] != -INFINITY) {   // wavefront pw contributed to this row block
+                const float* src = reinterpret_cast<const float*>(lds + pw * C::WAVE_LDS + C::TILE_BYTES);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) x[e] += wgt[pw][qb] * src[(4 * quad + e) * 64 + lane];
+              }
             }
-            M[qb] = mm; L[qb] = ll;
+            if (full) {
+              const float inv = 1.0f / L[qb];
+              const int64_t qrow = (int64_t)(r * 64 + qb * 32 + ln);
+              store_out4<BF16>(obase, qrow * prm.os[2] + 32 * db + 8 * i4 + 4 * g, prm.out_f32, x[0] * inv, x[1] * inv,
+                               x[2] * inv, x[3] * inv);
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) slot[(idx0 + e) * 64 + lane] = x[e];
+            }
           }
+          __syncthreads();
         }
+        if (w == 0 && g == 0) {
 #pragma unroll
-        for (int tq = 0; tq < C::QPW; ++tq) {
-          const int quad = w * C::QPW + tq;              // group of 4 registers within this round
-          const int idx0 = rd * C::R + 4 * quad;         // accumulator register index (db, qb, i16)
-          const int db = idx0 / 32, qb = (idx0 / 16) & 1, i4 = (idx0 & 15) / 4;
-          float x[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int pw = 0; pw < NW; ++pw) {
-            if (ml[(pw * 2 + 0) * 64] != -INFINITY) {   // wavefront pw contributed to this row block
-              const float* src = reinterpret_cast<const float*>(lds + pw * C::WAVE_LDS + C::TILE_BYTES);
-#pragma unroll
-              for (int e = 0; e < 4; ++e) x[e] += wgt[pw][qb] * src[(4 * quad + e) * 64 + lane];
-            }
-          }
-          if (full) {
-            const float inv = 1.0f / L[qb];
+          for (int qb = 0; qb < 2; ++qb) {
             const int64_t qrow = (int64_t)(r * 64 + qb * 32 + ln);
-            store_out4<BF16>(obase, qrow * prm.os[2] + 32 * db + 8 * i4 + 4 * g, prm.out_f32, x[0] * inv, x[1] * inv,
-                             x[2] * inv, x[3] * inv);
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) slot[(idx0 + e) * 64 + lane] = x[e];
-          }
-        }
-        __syncthreads();
-      }
-      if (w == 0 && g == 0) {
-#pragma unroll
-        for (int qb = 0; qb < 2; ++qb) {
-          const int64_t qrow = (int64_t)(r * 64 + qb * 32 + ln);
-          if (full) {
-            if (prm.lse != nullptr)
-              prm.lse[((int64_t)bh * prm.N) + qrow] = (M[qb] + __builtin_amdgcn_logf(L[qb])) * 0.6931471805599453f;
-          } else {
-            slot[64 * D + qb * 32 + ln] = M[qb];
-            slot[64 * D + 64 + qb * 32 + ln] = L[qb];
+            if (full) {
+              if (prm.lse != nullptr)
+                prm.lse[((int64_t)bh * prm.N) + qrow] = (M[qb] + __builtin_amdgcn_logf(L[qb])) * 0.6931471805599453f;
+            } else {
+              slot[64 * D + qb * 32 + ln] = M[qb];
+              slot[64 * D + 64 + qb * 32 + ln] = L[qb];
+            }
           }
         }
       }
+      first_seg = false;
+      t = seg_b;
+      ++r;
     }
-#ifdef EXP_TIMING
-    if (nseg == 0) Tc = __builtin_amdgcn_s_memrealtime();
-    ++nseg;
-#endif
-    first_seg = false;
-    t = seg_b;
-    ++r;
   }
-#ifdef EXP_TIMING
-  Td = __builtin_amdgcn_s_memrealtime();
-  if ((wg % 61) == 5 && lane == 0 && (w == 0 || w == 7))
-    printf("wg=%d w=%d mytiles=%d per tile: waitK %lld [1] %lld [2] %lld settle0 %lld waitV+dma %lld [3] %lld settle1 %lld [4] %lld\n", wg, w, ntile, tk[0]/ntile, tk[1]/ntile, tk[2]/ntile, tk[3]/ntile, tk[4]/ntile, tk[5]/ntile, tk[6]/ntile, tk[7]/ntile);
-  if ((wg % 61) == 5 && lane == 0 && (w == 0 || w == 7)) printf("wg=%d w=%d tiles=%d segs=%d | setup %lld | Q+first loads %lld | seg0 tiles %lld | seg0 merge %lld | rest %lld | total %lld (x10ns)\n", wg, w, g1 - g0, nseg, Ta - T0, Tq - Ta, Tb - Tq, Tc - Tb, Td - Tc, Td - T0);
-#endif
 }
 
 // One workgroup per row block: zero-fill empty rows, merge the partials of split rows.
@@ -652,17 +695,28 @@ size_t fwd_workspace_bytes(int B, int H, int N, int D) {
   return (size_t)B * H * W * 2 * partial_floats(D) * sizeof(float);
 }
 
+// With few row blocks per workgroup all wavefronts of a workgroup share one row block at a time
+// (K and V tiles are spread over them and the results merged); with many (>= 8 per workgroup) each
+// wavefront takes whole row blocks, which needs no merge and no second kernel.
+static bool rows_mode(const FwdParams& prm) { return prm.nb >= 8 * prm.W; }
+
 template <int D, bool BF16>
 static void launch_fwd_t(const FwdParams& prm, int BH, hipStream_t st) {
   using C = FwdCfg<D>;
   static bool configured = false;   // raising the dynamic LDS limit is idempotent
   if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<D, BF16>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<D, BF16, false>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<D, BF16, true>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
     configured = true;
   }
-  hipLaunchKernelGGL((fwd_kernel<D, BF16>), dim3(prm.W, BH), dim3(C::NW * 64), C::LDS_BYTES, st, prm);
-  hipLaunchKernelGGL((combine_kernel<D, BF16>), dim3(prm.nb, BH), dim3(64), 0, st, prm);
+  if (rows_mode(prm)) {
+    hipLaunchKernelGGL((fwd_kernel<D, BF16, true>), dim3(prm.W, BH), dim3(C::NW * 64), C::LDS_BYTES, st, prm);
+  } else {
+    hipLaunchKernelGGL((fwd_kernel<D, BF16, false>), dim3(prm.W, BH), dim3(C::NW * 64), C::LDS_BYTES, st, prm);
+    hipLaunchKernelGGL((combine_kernel<D, BF16>), dim3(prm.nb, BH), dim3(64), 0, st, prm);
+  }
 }
 
 int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,

@@ -79,13 +79,8 @@ typedef const int32_t __attribute__((address_space(4)))* cint_ptr_t;
 template <int D>
 __device__ __forceinline__ void tile_load_async(const unsigned short* tile, const unsigned (&off)[D / 8],
                                                 unsigned lds_addr) {
-#ifdef EXP_LOADSTEP
-#pragma unroll
-  for (int j = 0; j < D / 8; j += EXP_LOADSTEP)
-#else
 #pragma unroll
   for (int j = 0; j < D / 8; ++j)
-#endif
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :: "s"(lds_addr + j * 1024), "v"(off[j]), "s"(tile) : "memory", "m0");
 }

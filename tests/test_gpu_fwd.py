@@ -69,6 +69,34 @@ def test_empty_rows_and_all_false(dev):
     assert float(z.abs().max()) == 0.0                                       # fa2_custom_mask.py:49-51
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [64, 128])
+def test_many_heads_row_block_per_wavefront(dev, D, dtype):
+    """Many heads and many row blocks per workgroup: each wavefront runs whole row blocks (no merge,
+    no second kernel).  Covers empty row blocks at the start, inside and at the end of a head, a
+    head without kept tiles, and a head whose tiles sit in one row block."""
+    B, H, nb = 4, 64, 8
+    m = uniform_block_mask(B, H, nb, 0.4, 21)
+    m[0, 0, 0, :] = False
+    m[0, 1, 3:5, :] = False
+    m[0, 2, nb - 1, :] = False
+    m[1, 5] = False
+    m[2, 7] = False
+    m[2, 7, 4, :] = True
+    o = run_case(dev, B, H, nb * 64, D, dtype, m, 31)
+    assert float(o[1, 5].abs().max()) == 0.0 and float(o[0, 0, :64].abs().max()) == 0.0
+    run_case(dev, B, H, nb * 64, D, dtype, m, 31, out_fp32=True)
+
+
+def test_row_block_per_wavefront_several_workgroups_per_head(dev):
+    """64 heads x 32 row blocks: four workgroups per head, ranges cut inside row blocks."""
+    m = causal_block_mask(1, 1, 32, 0.6, 13)
+    run_case(dev, 2, 32, 2048, 64, torch.float16, m, 5)
+    m2 = uniform_block_mask(2, 32, 32, 0.15, 14)
+    m2[1, 3, 10:20, :] = False
+    run_case(dev, 2, 32, 2048, 64, torch.bfloat16, m2, 6, out_fp32=True)
+
+
 def test_dense_elementwise_mask_c2_small(dev):
     """Tile-constant elementwise mask gives the same result as its block mask."""
     import fa2_custom_mask as fm
