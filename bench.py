@@ -22,6 +22,10 @@ KEEPS = [0.05, 0.1, 0.25, 0.5, 1.0]
 PEAK_F16_TFLOPS = 2500.0     # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0
 SEED = 1234 + 2
+# HBM bytes of one keep-1.0 forward call (fwd_kernel + combine_kernel), from two rocprofv3 --pmc runs
+# (FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 after scaling by the readings of a 256 MiB device copy):
+# 108861 KiB fetched + 10643 KiB written.
+TRAFFIC_BYTES_PER_LAUNCH = (108861 + 10643) * 1024
 
 
 def tile_flops(kept):
@@ -40,17 +44,44 @@ def event_times(fn, iters, warmup, torch):
     return sorted(a.elapsed_time(b) for a, b in evs)       # ms
 
 
+def mfma_ceiling(torch, dev, iters=8192, launches=10):
+    """Sustained fp16 MFMA rate (TFLOP/s) of bsattn_mfma_rate_probe for two operand patterns."""
+    import ctypes
+    from fa2_custom_mask import _ext
+    lib = _ext.lib()
+    sink = torch.empty(512, dtype=torch.float32, device=dev)
+    st = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    g = torch.Generator().manual_seed(7)
+    out = {}
+    for name, ops in (("ones", torch.ones(4096, dtype=torch.float16)),
+                      ("randn", torch.randn(4096, generator=g).to(torch.float16))):
+        ops = ops.to(dev)
+        flops = ctypes.c_double()
+
+        def run():
+            _ext.check(lib.bsattn_mfma_rate_probe(ops.data_ptr(), iters, sink.data_ptr(),
+                                                  ctypes.byref(flops), st), "bsattn_mfma_rate_probe")
+        ts = event_times(run, launches, 3, torch)
+        out[name + "_tflops"] = round(flops.value / (ts[len(ts) // 2] * 1e-3) / 1e12, 1)
+    out["unit"] = "TFLOP/s"
+    out["what"] = "fp16 32x32x16 MFMA only, 2 wavefronts per SIMD, 4 accumulator chains, median of %d launches" % launches
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only-keep", type=float, default=None,
                     help="profiling aid: run only forward passes at this kept-tile ratio and exit")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="profiling aid: run a plain 256 MiB device copy a few times and exit "
                          "(reference reading for the FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--mfma-ceiling", action="store_true",
+                    help="measurement aid: the fp16 MFMA rate the GPU sustains with all-ones operands and "
+                         "with random operands (the clock depends on the data), then exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (heads / row blocks shard without "
@@ -71,6 +102,9 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes": 256 << 20, "copies": 5}))
+        return
+    if args.mfma_ceiling:
+        print(json.dumps(mfma_ceiling(torch, dev)))
         return
     g = torch.Generator().manual_seed(SEED)
     q, k, v = [torch.randn(1, 1, N, D, generator=g).to(torch.float16) for _ in range(3)]
@@ -111,7 +145,7 @@ def main():
     # ---- per-launch device time (HIP events on the launch stream), sweep of kept ratios ----
     sweep = {}
     for r in KEEPS:
-        ts = event_times(lambda: fwd(r), max(20, args.steps), 5, torch)
+        ts = event_times(lambda: fwd(r), min(200, max(20, args.steps)), 5, torch)
         avg, med = sum(ts) / len(ts), ts[len(ts) // 2]
         sweep[str(r)] = {"kept_tiles": kept[r], "ms_avg": round(avg, 5), "ms_median": round(med, 5),
                          "tflops": round(tile_flops(kept[r]) / (med * 1e-3) / 1e12, 2),
@@ -149,8 +183,8 @@ def main():
                             "block_mask_ms": round(ts_b[len(ts_b) // 2], 5)},
         "parity_max_abs_vs_oracle": parity,
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": None,
-                     "kernel": "fwd_kernel<64,false> + combine_kernel<64,false> (one bsattn_fwd call)",
+                     "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
+                     "kernel": "fwd_kernel<64,false,false> (one bsattn_fwd call)",
                      "algorithmic_flops_per_launch": tile_flops(kept[1.0])},
     }
     if not args.no_cpu:

@@ -1,14 +1,18 @@
 // Block-sparse FlashAttention-2 forward for gfx950.
 //
 // Work decomposition.  The kept tiles of one head form a list in row-major order; it is cut
-// into W equal contiguous ranges, one per workgroup, regardless of row boundaries (W depends on
-// shapes only, so no host synchronisation on the mask content is needed).  A workgroup walks
+// into W contiguous ranges, one per workgroup, regardless of row boundaries (W depends on
+// shapes only, so no host synchronisation on the mask content is needed; where two workgroups
+// share a compute unit the first-comer's range is longer, see fwd_split.h).  A workgroup walks
 // its range row block by row block; the kept tiles of the current row block that fall inside
-// the range are split evenly over the workgroup's wavefronts, each of which runs the online
-// softmax over its share with private LDS tile buffers, and the per-wavefront results
-// (acc, m, l) are merged through LDS.  A row block that lies completely inside the range is
-// normalised and written straight to O; a row block shared with a neighbouring workgroup is
-// written as an unnormalised partial and merged by combine_kernel.
+// the range are handed to the workgroup's wavefronts one at a time, each wavefront runs the
+// online softmax over the tiles it gets with private LDS tile buffers, and the per-wavefront
+// results (acc, m, l) are merged through LDS.  A row block that lies completely inside the
+// range is normalised and written straight to O.  A row block cut by range boundaries is
+// finished by the workgroup that holds its first tiles: the others publish unnormalised parts
+// in the workspace (device-scope stores, then a flag), and it pulls them when it gets there.
+// With many row blocks per workgroup (many heads) each wavefront takes whole row blocks
+// instead, and nothing is merged.
 //
 // Per tile a wavefront computes S^T = K Q^T (keys along MFMA rows, queries along lanes), so
 // that one lane owns one query: softmax statistics are in-lane reductions plus a single
@@ -19,6 +23,8 @@
 // statistics, P rounded to 16 bits for the second product), with two changes that keep the
 // vector ALU out of the way of the matrix cores: the softmax scale is folded into Q, and the
 // running maximum is replaced by a reference exponent that is only moved when needed.
+#include <atomic>
+#include <chrono>
 #include "common.h"
 #include "fwd_split.h"
 #include "kernel_util.h"
@@ -28,8 +34,11 @@ namespace bsattn {
 struct FwdParams {
   const void* q; const void* k; const void* v; void* o; float* lse;
   const int32_t* row_ptr; const int32_t* col_idx;
-  float* ws;
+  float* ws;                       // partial slots of row blocks shared between workgroups
+  unsigned long long* flags;       // one per slot: holds `epoch` once the slot's part is complete
+  unsigned long long epoch;        // distinguishes this launch's flags from stale contents
   int B, H, N, nb, Bm, Hm, W;   // W: workgroups per head
+  int first_ids;                // workgroups with a linear id below this are the first on their compute unit
   int out_f32;
   float qk_scale;  // sm_scale * log2(e)
   int64_t qs[3], ks[3], vs[3], os[3];
@@ -98,9 +107,22 @@ __device__ __forceinline__ void recentre(floatx16& s0, floatx16& s1, floatx16 (&
   }
 }
 
-// Number of wavefronts of a workgroup: 2 per SIMD at D=64 (256 VGPRs each), 1 per SIMD at D=128.
+
+// Partial results cross workgroups (and the L2 slices of different XCDs) inside one launch:
+// they are written and read with device-scope accesses, which go to the point of coherence.
+__device__ __forceinline__ void coherent_store(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float coherent_load(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// A workgroup is four wavefronts, one per SIMD.  At D=64 a wavefront needs 256 registers and two
+// workgroups share a compute unit (while one merges or waits for its first tiles the other computes);
+// at D=128 a wavefront needs all 512 registers of its SIMD.
 template <int D> struct FwdCfg {
-  static constexpr int NW = D == 64 ? 8 : 4;
+  static constexpr int NW = 4;
+  static constexpr int WG_PER_CU = D == 64 ? 2 : 1;
   static constexpr int TILE_BYTES = 64 * 2 * D;             // one K or V tile in LDS
   static constexpr int WAVE_LDS = 2 * TILE_BYTES;           // K buffer + V buffer
   static constexpr int ML_BYTES = NW * 2 * 64 * 4 + 64;     // exchange of (m, l) per query + the tile counter
@@ -112,7 +134,7 @@ template <int D> struct FwdCfg {
 };
 
 template <int D, bool BF16, bool ROWS>
-__global__ __launch_bounds__(FwdCfg<D>::NW * 64)
+__global__ __launch_bounds__(FwdCfg<D>::NW * 64, FwdCfg<D>::WG_PER_CU)
 void fwd_kernel(const FwdParams prm) {
   using C = FwdCfg<D>;
   constexpr int NW = C::NW;
@@ -126,18 +148,35 @@ void fwd_kernel(const FwdParams prm) {
   const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int ln = lane & 31, g = lane >> 5;
-  const int wg = blockIdx.x, bh = blockIdx.y;
+  // linear id -> (head, range): heads interleaved, so that every head gets its share of the
+  // workgroups that are first on their compute unit
+  const int BH = prm.B * prm.H;
+  const int bh = blockIdx.x % BH, wg = blockIdx.x / BH;
   const int b = bh / prm.H, h = bh % prm.H;
   const int mh = (prm.Bm > 1 ? b : 0) * prm.Hm + (prm.Hm > 1 ? h : 0);
   const int nb = prm.nb;
   // the lists are read-only for the whole launch: constant address space => scalar loads
   const cint_ptr_t rp = (cint_ptr_t)(uintptr_t)(prm.row_ptr + (int64_t)mh * nb);
   const cint_ptr_t cols = (cint_ptr_t)(uintptr_t)prm.col_idx;
-  const HeadSplit hs = head_split(rp, nb, prm.W, NW);
-  // a head without kept tiles: the row-per-wavefront driver still has to write its zeros
-  if (wg >= (ROWS && hs.T == 0 ? 1 : hs.Peff)) return;
+  const HeadSplit hs = head_split(rp, nb, prm.W, NW, prm.first_ids > bh ? (prm.first_ids - bh + BH - 1) / BH : 0);
+  // a head without kept tiles still needs its zeros: workgroup 0 writes them
+  const int Pact = hs.T == 0 ? 1 : hs.Peff;
+  if (wg >= Pact) return;
   const int g0 = hs.T > 0 ? split_begin(hs, wg) : hs.lo, g1 = hs.T > 0 ? split_begin(hs, wg + 1) : hs.lo;
-  if (!ROWS && g0 >= g1) return;
+  if constexpr (!ROWS) {
+    // Row blocks without kept tiles belong to no range: they are dealt round-robin, and the
+    // workgroup writes O = 0, lse = -inf for its share.
+    for (int r0 = wg; r0 < nb; r0 += Pact) {
+      if (rp[r0 + 1] > rp[r0]) continue;
+      void* ob = out_base(prm, b, h);
+      for (int i = threadIdx.x; i < 64 * (D / 4); i += NW * 64) {
+        const int64_t qrow = (int64_t)r0 * 64 + i / (D / 4);
+        store_out4<BF16>(ob, qrow * prm.os[2] + 4 * (i % (D / 4)), prm.out_f32, 0.f, 0.f, 0.f, 0.f);
+      }
+      if (prm.lse != nullptr && threadIdx.x < 64) prm.lse[(int64_t)bh * prm.N + (int64_t)r0 * 64 + threadIdx.x] = -INFINITY;
+    }
+    if (g0 >= g1) return;
+  }
 
   unsigned char* lds_k = lds + w * C::WAVE_LDS;
   unsigned char* lds_v = lds_k + C::TILE_BYTES;
@@ -465,7 +504,6 @@ void fwd_kernel(const FwdParams prm) {
     int cur = g0 + w, nxt = g0 + NW + w;      // the first two rounds are fixed
     int cb_nxt = nxt < g1 ? __builtin_amdgcn_readfirstlane(col_of(nxt)) : 0;   // column block of tile nxt
     int kdone = -1, vdone = -1;
-    bool first_seg = true;
     int t = g0;
     while (t < g1) {
       const int row_s = rp[r], row_e = rp[r + 1];
@@ -495,7 +533,6 @@ void fwd_kernel(const FwdParams prm) {
           cb_nxt = __builtin_amdgcn_readfirstlane(cb_nn_v);
         }  // tiles of this wavefront
       }
-
       // ---- merge the wavefronts' results of this row block through LDS ----
       // Each wavefront publishes (m, l) per query and, round by round, R accumulator registers in
       // its own V buffer ([register][lane] floats); in every round each wavefront reduces QPW
@@ -512,14 +549,22 @@ void fwd_kernel(const FwdParams prm) {
             ml[(w * 2 + 1) * 64 + qb * 32 + ln] = mine ? lsum[qb] : 0.f;
           }
         }
-        const bool full = (seg_a == row_s) && (seg_b == row_e);
+        // A row block cut by range boundaries is finished by the workgroup that holds its first
+        // tiles (for that workgroup it is the last row block of its range): the other workgroups
+        // publish their parts (for them it is the first row block of their ranges, so the parts
+        // are ready early), and the finishing workgroup pulls them.
+        const bool has_head = seg_a == row_s, has_tail = seg_b == row_e;
+        const bool full = has_head && has_tail, publish = !has_head, pull = has_head && !has_tail;
         float wgt[NW][2];   // weight of wavefront p's partial for this lane's query of block qb
         float M[2], L[2];
-        float* slot = prm.ws + ((((int64_t)bh * prm.W + wg) * 2) + (first_seg ? 0 : 1)) * partial_floats(D);
+        float keep[C::ROUNDS][C::QPW][4];   // this wavefront's share of the merged accumulator (pull)
+        float* slot = prm.ws + ((int64_t)bh * prm.W + wg) * partial_floats(D);
         void* obase = out_base(prm, b, h);
 #pragma unroll
         for (int rd = 0; rd < C::ROUNDS; ++rd) {
-          if (mine) {
+          {
+            // every wavefront writes (one without tiles of this row block holds zeros), 4 bytes per
+            // lane and instruction: wider LDS writes are much slower per byte on this hardware
             float* own = reinterpret_cast<float*>(lds_v);
 #pragma unroll
             for (int e = 0; e < C::R; ++e) {
@@ -553,146 +598,150 @@ void fwd_kernel(const FwdParams prm) {
             float x[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int pw = 0; pw < NW; ++pw) {
-              if (ml[(pw * 2 + 0) * 64] != -INFINITY) {   // wavefront pw contributed to this row block
-                const float* src = reinterpret_cast<const float*>(lds + pw * C::WAVE_LDS + C::TILE_BYTES);
+              const float* src = reinterpret_cast<const float*>(lds + pw * C::WAVE_LDS + C::TILE_BYTES);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) x[e] += wgt[pw][qb] * src[(4 * quad + e) * 64 + lane];
-              }
+              for (int e = 0; e < 4; ++e) x[e] += wgt[pw][qb] * src[(4 * quad + e) * 64 + lane];
             }
             if (full) {
               const float inv = 1.0f / L[qb];
               const int64_t qrow = (int64_t)(r * 64 + qb * 32 + ln);
               store_out4<BF16>(obase, qrow * prm.os[2] + 32 * db + 8 * i4 + 4 * g, prm.out_f32, x[0] * inv, x[1] * inv,
                                x[2] * inv, x[3] * inv);
-            } else {
+            } else if (publish) {
 #pragma unroll
-              for (int e = 0; e < 4; ++e) slot[(idx0 + e) * 64 + lane] = x[e];
+              for (int e = 0; e < 4; ++e) coherent_store(slot + (idx0 + e) * 64 + lane, x[e]);
             }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) keep[rd][tq][e] = x[e];
           }
           __syncthreads();
         }
-        if (w == 0 && g == 0) {
+        if (full) {
+          if (w == 0 && g == 0 && prm.lse != nullptr) {
 #pragma unroll
-          for (int qb = 0; qb < 2; ++qb) {
-            const int64_t qrow = (int64_t)(r * 64 + qb * 32 + ln);
-            if (full) {
-              if (prm.lse != nullptr)
-                prm.lse[((int64_t)bh * prm.N) + qrow] = (M[qb] + __builtin_amdgcn_logf(L[qb])) * 0.6931471805599453f;
-            } else {
-              slot[64 * D + qb * 32 + ln] = M[qb];
-              slot[64 * D + 64 + qb * 32 + ln] = L[qb];
+            for (int qb = 0; qb < 2; ++qb)
+              prm.lse[((int64_t)bh * prm.N) + (int64_t)(r * 64 + qb * 32 + ln)] =
+                  (M[qb] + __builtin_amdgcn_logf(L[qb])) * 0.6931471805599453f;
+          }
+        } else if (publish) {
+          if (w == 0 && g == 0) {
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb) {
+              coherent_store(slot + 64 * D + qb * 32 + ln, M[qb]);
+              coherent_store(slot + 64 * D + 64 + qb * 32 + ln, L[qb]);
             }
           }
+          // the flag goes up once every wavefront's stores have been acknowledged
+          wait_vm<0>();
+          __syncthreads();
+          if (threadIdx.x == 0)
+            __hip_atomic_store(prm.flags + (int64_t)bh * prm.W + wg, prm.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+          // pull the parts of the workgroups wg+1 .. pl and finish the row block
+          const int pl_ = split_of_tile(hs, row_e - 1);
+          bool ok = true;
+          for (int p = wg + 1; p <= pl_; ++p) {
+            unsigned long long* fl = prm.flags + (int64_t)bh * prm.W + p;
+            // The wait is bounded (about 0.2 s of the 100 MHz counter): a part that never arrives
+            // turns the row block into NaNs instead of a hang.
+            const long long t_start = __builtin_amdgcn_s_memrealtime();
+            while (__hip_atomic_load(fl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != prm.epoch) {
+              if (__builtin_amdgcn_s_memrealtime() - t_start > 20000000ll) { ok = false; break; }
+              __builtin_amdgcn_s_sleep(4);
+            }
+            const float* sp = prm.ws + ((int64_t)bh * prm.W + p) * partial_floats(D);
+            float sc_own[2], sc_p[2];
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb) {
+              const float mp = coherent_load(sp + 64 * D + qb * 32 + ln), lp = coherent_load(sp + 64 * D + 64 + qb * 32 + ln);
+              const float mn = fmaxf(M[qb], mp);
+              sc_own[qb] = __builtin_amdgcn_exp2f(M[qb] - mn);
+              sc_p[qb] = __builtin_amdgcn_exp2f(mp - mn);
+              L[qb] = L[qb] * sc_own[qb] + lp * sc_p[qb];
+              M[qb] = mn;
+            }
+#pragma unroll
+            for (int rd = 0; rd < C::ROUNDS; ++rd)
+#pragma unroll
+              for (int tq = 0; tq < C::QPW; ++tq) {
+                const int idx0 = rd * C::R + 4 * (w * C::QPW + tq);
+                const int qb = (idx0 / 16) & 1;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                  keep[rd][tq][e] = keep[rd][tq][e] * sc_own[qb] + sc_p[qb] * coherent_load(sp + (idx0 + e) * 64 + lane);
+              }
+          }
+          const float bad = ok ? 0.f : __builtin_nanf("");
+#pragma unroll
+          for (int rd = 0; rd < C::ROUNDS; ++rd)
+#pragma unroll
+            for (int tq = 0; tq < C::QPW; ++tq) {
+              const int idx0 = rd * C::R + 4 * (w * C::QPW + tq);
+              const int db = idx0 / 32, qb = (idx0 / 16) & 1, i4 = (idx0 & 15) / 4;
+              const float inv = 1.0f / L[qb];
+              const int64_t qrow = (int64_t)(r * 64 + qb * 32 + ln);
+              store_out4<BF16>(obase, qrow * prm.os[2] + 32 * db + 8 * i4 + 4 * g, prm.out_f32,
+                               keep[rd][tq][0] * inv + bad, keep[rd][tq][1] * inv + bad, keep[rd][tq][2] * inv + bad,
+                               keep[rd][tq][3] * inv + bad);
+            }
+          if (w == 0 && g == 0 && prm.lse != nullptr) {
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb)
+              prm.lse[((int64_t)bh * prm.N) + (int64_t)(r * 64 + qb * 32 + ln)] =
+                  (M[qb] + __builtin_amdgcn_logf(L[qb])) * 0.6931471805599453f + bad;
+          }
+          // every wavefront has read the flags: put them back to zero, so that a replay of this
+          // launch (same epoch) does not take this launch's parts for its own
+          __syncthreads();
+          if (threadIdx.x == 0)
+            for (int p = wg + 1; p <= pl_; ++p)
+              __hip_atomic_store(prm.flags + (int64_t)bh * prm.W + p, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
       }
-      first_seg = false;
       t = seg_b;
       ++r;
     }
   }
 }
 
-// One workgroup per row block: zero-fill empty rows, merge the partials of split rows.
-template <int D, bool BF16>
-__global__ __launch_bounds__(64) void combine_kernel(const FwdParams prm) {
-  constexpr int DB = D / 32;
-  const int lane = threadIdx.x, ln = lane & 31, g = lane >> 5;
-  const int m = blockIdx.x, bh = blockIdx.y;
-  const int b = bh / prm.H, h = bh % prm.H;
-  const int mh = (prm.Bm > 1 ? b : 0) * prm.Hm + (prm.Hm > 1 ? h : 0);
-  const int nb = prm.nb;
-  const int32_t* rp = prm.row_ptr + (int64_t)mh * nb;
-  const int rs = rp[m], re = rp[m + 1];
-  float acc[DB][2][16];
-  float M[2] = {-INFINITY, -INFINITY}, L[2] = {0.f, 0.f};
-#pragma unroll
-  for (int db = 0; db < DB; ++db)
-#pragma unroll
-    for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[db][qb][i] = 0.f;
-  if (re > rs) {
-    const HeadSplit hs = head_split(rp, nb, prm.W, FwdCfg<D>::NW);
-    const int pf = split_of_tile(hs, rs), pl = split_of_tile(hs, re - 1);
-    if (pf == pl) return;  // the whole row lies in one range: already final
-    for (int p = pf; p <= pl; ++p) {
-      const int pt0 = split_begin(hs, p);
-      const int slot_id = (pt0 >= rs) ? 0 : 1;  // is this the first row block of range p?
-      const float* slot = prm.ws + ((((int64_t)bh * prm.W + p) * 2) + slot_id) * partial_floats(D);
-      float mp[2], lp[2];
-#pragma unroll
-      for (int qb = 0; qb < 2; ++qb) { mp[qb] = slot[64 * D + qb * 32 + ln]; lp[qb] = slot[64 * D + 64 + qb * 32 + ln]; }
-#pragma unroll
-      for (int qb = 0; qb < 2; ++qb) {
-        const float mn = fmaxf(M[qb], mp[qb]);
-        const float so = __builtin_amdgcn_exp2f(M[qb] - mn), sn = __builtin_amdgcn_exp2f(mp[qb] - mn);
-        L[qb] = L[qb] * so + lp[qb] * sn;
-        M[qb] = mn;
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-          for (int i = 0; i < 16; ++i)
-            acc[db][qb][i] = acc[db][qb][i] * so + slot[((db * 2 + qb) * 16 + i) * 64 + lane] * sn;
-      }
-    }
-  }
-#pragma unroll
-  for (int qb = 0; qb < 2; ++qb) {
-    const float inv = re > rs ? 1.0f / L[qb] : 0.f;
-    const int64_t qrow = (int64_t)(m * 64 + qb * 32 + ln);
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int i4 = 0; i4 < 4; ++i4) {
-        const int d0 = 32 * db + 8 * i4 + 4 * g;
-        float x[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) x[e] = acc[db][qb][4 * i4 + e] * inv;
-        if (prm.out_f32) {
-          float* orow = (float*)prm.o + b * prm.os[0] + h * prm.os[1] + qrow * prm.os[2];
-          floatx4 w = {x[0], x[1], x[2], x[3]};
-          *reinterpret_cast<floatx4*>(orow + d0) = w;
-        } else {
-          unsigned short* orow = (unsigned short*)prm.o + b * prm.os[0] + h * prm.os[1] + qrow * prm.os[2];
-          uintx2 w;
-#pragma unroll
-          for (int e = 0; e < 2; ++e) {
-            if constexpr (BF16) {
-              typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
-              bf2 hv = {(__bf16)x[2 * e], (__bf16)x[2 * e + 1]};
-              w[e] = __builtin_bit_cast(unsigned int, hv);
-            } else {
-              typedef _Float16 half2v __attribute__((ext_vector_type(2)));
-              half2v hv = {(_Float16)x[2 * e], (_Float16)x[2 * e + 1]};
-              w[e] = __builtin_bit_cast(unsigned int, hv);
-            }
-          }
-          *reinterpret_cast<uintx2*>(orow + d0) = w;
-        }
-      }
-    if (prm.lse != nullptr && g == 0)
-      prm.lse[((int64_t)bh * prm.N) + qrow] =
-          re > rs ? (M[qb] + __builtin_amdgcn_logf(L[qb])) * 0.6931471805599453f : -INFINITY;
-  }
+// A 48-bit number that differs from launch to launch (and, through its start value, from process
+// to process); never zero.
+static unsigned long long next_epoch() {
+  static std::atomic<unsigned long long> counter{
+      (unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count() * 0x9E3779B97F4A7C15ull};
+  unsigned long long e;
+  do { e = counter.fetch_add(1) & 0xffffffffffffull; } while (e == 0);
+  return e;
 }
 
-static int groups_per_head(int B, int H, int nb) {
+static int compute_units() {
   int dev = 0, cus = 256;
   if (hipGetDevice(&dev) == hipSuccess) {
     int v = 0;
     if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
   }
-  int64_t W = cus / ((int64_t)B * H);   // one resident workgroup per CU
+  return cus;
+}
+
+static int groups_per_head(int B, int H, int nb, int D) {
+  const int cus = compute_units();
+  const int per_cu = D == 64 ? FwdCfg<64>::WG_PER_CU : FwdCfg<128>::WG_PER_CU;
+  int64_t W = (int64_t)cus * per_cu / ((int64_t)B * H);   // as many workgroups as are resident at once
   const int64_t cap = (int64_t)nb * nb;
   if (W > cap) W = cap;
   if (W < 1) W = 1;
   return (int)W;
 }
 
+// workspace: partial slots [B*H][W][partial_floats] (fp32), then their flags [B*H][W] (64 bit)
+static size_t slots_bytes(int B, int H, int W, int D) {
+  return (size_t)B * H * W * partial_floats(D) * sizeof(float);
+}
+
 size_t fwd_workspace_bytes(int B, int H, int N, int D) {
   const int nb = N / 64;
-  const int W = groups_per_head(B, H, nb);
-  return (size_t)B * H * W * 2 * partial_floats(D) * sizeof(float);
+  const int W = groups_per_head(B, H, nb, D);
+  return slots_bytes(B, H, W, D) + (size_t)B * H * W * sizeof(unsigned long long);
 }
 
 // With few row blocks per workgroup all wavefronts of a workgroup share one row block at a time
@@ -712,10 +761,9 @@ static void launch_fwd_t(const FwdParams& prm, int BH, hipStream_t st) {
     configured = true;
   }
   if (rows_mode(prm)) {
-    hipLaunchKernelGGL((fwd_kernel<D, BF16, true>), dim3(prm.W, BH), dim3(C::NW * 64), C::LDS_BYTES, st, prm);
+    hipLaunchKernelGGL((fwd_kernel<D, BF16, true>), dim3(prm.W * BH), dim3(C::NW * 64), C::LDS_BYTES, st, prm);
   } else {
-    hipLaunchKernelGGL((fwd_kernel<D, BF16, false>), dim3(prm.W, BH), dim3(C::NW * 64), C::LDS_BYTES, st, prm);
-    hipLaunchKernelGGL((combine_kernel<D, BF16>), dim3(prm.nb, BH), dim3(64), 0, st, prm);
+    hipLaunchKernelGGL((fwd_kernel<D, BF16, false>), dim3(prm.W * BH), dim3(C::NW * 64), C::LDS_BYTES, st, prm);
   }
 }
 
@@ -726,7 +774,11 @@ int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
   prm.q = q; prm.k = k; prm.v = v; prm.o = o; prm.lse = lse;
   prm.row_ptr = row_ptr; prm.col_idx = col_idx; prm.ws = (float*)ws;
   prm.B = s.B; prm.H = s.H; prm.N = s.N; prm.nb = s.N / 64; prm.Bm = s.Bm; prm.Hm = s.Hm;
-  prm.W = groups_per_head(s.B, s.H, prm.nb);
+  prm.W = groups_per_head(s.B, s.H, prm.nb, s.D);
+  // with two workgroups per compute unit the first-comers are faster: tell the kernel which they are
+  prm.first_ids = (s.D == 64 ? FwdCfg<64>::WG_PER_CU : FwdCfg<128>::WG_PER_CU) > 1 ? compute_units() : 0;
+  prm.flags = (unsigned long long*)((char*)ws + slots_bytes(s.B, s.H, prm.W, s.D));
+  prm.epoch = next_epoch();
   prm.out_f32 = s.out_dtype == BSATTN_F32;
   prm.qk_scale = s.sm_scale * 1.4426950408889634f;
   for (int i = 0; i < 3; ++i) { prm.qs[i] = s.qs[i]; prm.ks[i] = s.ks[i]; prm.vs[i] = s.vs[i]; prm.os[i] = s.os[i]; }

@@ -37,9 +37,10 @@ def f32(x):
     return x.detach().float().cpu().numpy()
 
 
-def same_up_to_rounding(a, b, rel=2.0 ** -10, abs_=1e-4):
-    """Two runs of the forward may sum a row's tiles in a different order (tiles are handed to
-    wavefronts dynamically): equal up to one rounding step of the 16-bit output."""
+def same_up_to_rounding(a, b, rel=2.0 ** -9, abs_=3e-4):
+    """Two runs of the forward may split a row's tiles differently over wavefronts (tiles are handed
+    out dynamically), which changes the summation order and the reference exponents the fp16
+    probabilities are rounded against: equal up to two rounding steps of the 16-bit output."""
     a = a.detach().float().cpu().numpy() if isinstance(a, torch.Tensor) else np.asarray(a, dtype=np.float32)
     b = b.detach().float().cpu().numpy() if isinstance(b, torch.Tensor) else np.asarray(b, dtype=np.float32)
     return bool(np.all(np.abs(a - b) <= rel * np.abs(b) + abs_))
