@@ -22,10 +22,10 @@ KEEPS = [0.05, 0.1, 0.25, 0.5, 1.0]
 PEAK_F16_TFLOPS = 2500.0     # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0
 SEED = 1234 + 2
-# HBM bytes of one keep-1.0 forward call (fwd_kernel + combine_kernel), from two rocprofv3 --pmc runs
-# (FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 after scaling by the readings of a 256 MiB device copy):
-# 108861 KiB fetched + 10643 KiB written.
-TRAFFIC_BYTES_PER_LAUNCH = (108861 + 10643) * 1024
+# HBM-side bytes of one keep-1.0 forward launch, from two rocprofv3 --pmc runs (FETCH_SIZE x 2.0 and
+# WRITE_SIZE x 1.0 after scaling by the readings of a 256 MiB device copy): 226863 KiB fetched +
+# 18899 KiB written.
+TRAFFIC_BYTES_PER_LAUNCH = (226863 + 18899) * 1024
 
 
 def tile_flops(kept):
