@@ -44,6 +44,31 @@ def event_times(fn, iters, warmup, torch):
     return sorted(a.elapsed_time(b) for a, b in evs)       # ms
 
 
+def fwd_bwd_c5(torch, dev, fm, steps, warmup):
+    """HIP-event times of one forward call and one backward call at configs[4]."""
+    from fa2_custom_mask import fa2_custom_mask as host
+    B, H, Nc, Dc = 2, 16, 8192, 128
+    nbc = Nc // TILE
+    g = torch.Generator().manual_seed(1238)
+    q, k, v, do = [torch.randn(B, H, Nc, Dc, generator=g).to(torch.bfloat16).to(dev) for _ in range(4)]
+    m = (torch.rand(1, 1, nbc, nbc, generator=g) < 0.25) | torch.eye(nbc, dtype=torch.bool)
+    m = torch.tril(m.reshape(nbc, nbc)).reshape(1, 1, nbc, nbc).to(dev)
+    lists = fm.block_mask_to_lists(m)
+    lists_t = fm.block_mask_to_lists(m, transpose=True)
+    tiles = int(lists.counts[1]) * B * H
+    sc = 1.0 / Dc ** 0.5
+    o, lse = host._forward(q, k, v, lists, sc, torch.bfloat16, True)
+    tf = event_times(lambda: host._forward(q, k, v, lists, sc, torch.bfloat16, True), steps, warmup, torch)
+    tb = event_times(lambda: host._backward(q, k, v, o, do, lse, lists, lists_t, sc, torch.bfloat16), steps, warmup, torch)
+    mf, mb = tf[len(tf) // 2], tb[len(tb) // 2]
+    ff, fb = tiles * 4.0 * TILE * TILE * Dc, tiles * 10.0 * TILE * TILE * Dc
+    return {"workload": "BASELINE configs[4]: fwd+bwd B=2 H=16 N=8192 D=128 bf16, block-causal keep 0.25 shared mask",
+            "kept_tiles": tiles, "fwd_ms": round(mf, 5), "fwd_tflops": round(ff / mf / 1e9, 1),
+            "bwd_ms": round(mb, 5), "bwd_tflops": round(fb / mb / 1e9, 1),
+            "frac_mfma_peak": {"fwd": round(ff / mf / 1e9 / PEAK_F16_TFLOPS, 4), "bwd": round(fb / mb / 1e9 / PEAK_F16_TFLOPS, 4)},
+            "note": "times include the per-call output/workspace allocation of the host wrapper"}
+
+
 def mfma_ceiling(torch, dev, iters=8192, launches=10):
     """Sustained fp16 MFMA rate (TFLOP/s) of bsattn_mfma_rate_probe for two operand patterns."""
     import ctypes
@@ -79,6 +104,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="profiling aid: run a plain 256 MiB device copy a few times and exit "
                          "(reference reading for the FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--fwd-bwd", action="store_true",
+                    help="measurement aid: forward and backward at BASELINE configs[4] (B=2 H=16 N=8192 D=128 bf16, "
+                         "block-causal mask with keep 0.25 shared by all heads), then exit")
     ap.add_argument("--mfma-ceiling", action="store_true",
                     help="measurement aid: the fp16 MFMA rate the GPU sustains with all-ones operands and "
                          "with random operands (the clock depends on the data), then exit")
@@ -105,6 +133,9 @@ def main():
         return
     if args.mfma_ceiling:
         print(json.dumps(mfma_ceiling(torch, dev)))
+        return
+    if args.fwd_bwd:
+        print(json.dumps(fwd_bwd_c5(torch, dev, fm, min(args.steps, 50), min(args.warmup, 5))))
         return
     g = torch.Generator().manual_seed(SEED)
     q, k, v = [torch.randn(1, 1, N, D, generator=g).to(torch.float16) for _ in range(3)]
@@ -182,6 +213,7 @@ def main():
                             "frac_hbm_peak": round(pre_bytes / (pre_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                             "block_mask_ms": round(ts_b[len(ts_b) // 2], 5)},
         "parity_max_abs_vs_oracle": parity,
+        "fwd_bwd_configs4": fwd_bwd_c5(torch, dev, fm, 20, 3),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
                      "kernel": "fwd_kernel<64,false,false> (one bsattn_fwd call)",

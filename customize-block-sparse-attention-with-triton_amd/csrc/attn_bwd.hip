@@ -141,6 +141,18 @@ __device__ __forceinline__ floatx16 zero16() {
   return z;
 }
 
+
+// Workgroup -> (head, block) for the walking kernels.  Workgroups go to the 8 XCDs round-robin by
+// linear id, and each XCD has its own L2: heads are taken in groups of 8, head i of a group on
+// XCD i, so that the tiles a head's workgroups walk over (K and V, or Q and dO, of that head) are
+// shared in one L2 instead of being fetched into all of them.
+__device__ __forceinline__ void head_and_block(int L, int BH, int nb, int& bh, int& blk) {
+  const int grp = L / (8 * nb), l = L - grp * 8 * nb;
+  const int hg = BH - 8 * grp < 8 ? BH - 8 * grp : 8;     // heads in this group
+  bh = 8 * grp + l % hg;
+  blk = l / hg;          // >= nb for the padding of an incomplete last group
+}
+
 // ---------------------------------------------------------------------------------------
 // dQ: workgroup = row block m, wavefront wv owns queries 64m + 32wv + ln
 // ---------------------------------------------------------------------------------------
@@ -152,8 +164,11 @@ __global__ __launch_bounds__(128) void dq_kernel(const BwdParams prm) {
   const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int ln = lane & 31, g = lane >> 5;
   const int nb = prm.nb;
-  const int m = nb - 1 - blockIdx.x;          // long rows of block-causal masks first
-  const int bh = blockIdx.y, b = bh / prm.H, h = bh % prm.H;
+  int bh, blk;
+  head_and_block(blockIdx.x, prm.B * prm.H, nb, bh, blk);
+  if (blk >= nb) return;
+  const int m = nb - 1 - blk;                 // long rows of block-causal masks first
+  const int b = bh / prm.H, h = bh % prm.H;
   const int mh = (prm.Bm > 1 ? b : 0) * prm.Hm + (prm.Hm > 1 ? h : 0);
   const cint_ptr_t rp = (cint_ptr_t)(uintptr_t)(prm.row_ptr + (int64_t)mh * nb);
   const cint_ptr_t cols = (cint_ptr_t)(uintptr_t)prm.col_idx;
@@ -197,6 +212,17 @@ __global__ __launch_bounds__(128) void dq_kernel(const BwdParams prm) {
     const unsigned char* kt = lds + stage * C::STAGE_BYTES;
     const unsigned char* vt = kt + C::TILE_BYTES;
 
+    // All operand fragments of a block of MFMAs are read from LDS before the block starts: a read
+    // issued next to the MFMA that consumes it costs a full LDS latency per MFMA.
+    uintx4 fk[2][KS], fv[2][KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        fk[kb][s] = frag_rows<D>(kt, 32 * kb, s, ln, g);
+        fv[kb][s] = frag_rows<D>(vt, 32 * kb, s, ln, g);
+      }
+    __builtin_amdgcn_sched_barrier(0);
     floatx16 sacc[2], dpacc[2];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) { sacc[kb] = zero16(); dpacc[kb] = zero16(); }
@@ -204,9 +230,17 @@ __global__ __launch_bounds__(128) void dq_kernel(const BwdParams prm) {
     for (int s = 0; s < KS; ++s)
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
-        sacc[kb] = mfma_qk<BF16>(frag_rows<D>(kt, 32 * kb, s, ln, g), qfr[s], sacc[kb]);      // S^T = K Q^T
-        dpacc[kb] = mfma_qk<BF16>(frag_rows<D>(vt, 32 * kb, s, ln, g), dofr[s], dpacc[kb]);   // dP^T = V dO^T
+        sacc[kb] = mfma_qk<BF16>(fk[kb][s], qfr[s], sacc[kb]);      // S^T = K Q^T
+        dpacc[kb] = mfma_qk<BF16>(fv[kb][s], dofr[s], dpacc[kb]);   // dP^T = V dO^T
       }
+    __builtin_amdgcn_sched_barrier(0);
+    // K^T fragments of the second product, read under the exponentials below
+    uintx4 fkt[4][DB];
+#pragma unroll
+    for (int ts = 0; ts < 4; ++ts)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) fkt[ts][db] = frag_cols<D, BF16>(kt, db, ts, lane);
+    __builtin_amdgcn_sched_barrier(0);
     // dS^T = P^T * (dP^T - delta), this lane's query; packed as operand slices of 16 keys
     uintx4 dsf[4];
 #pragma unroll
@@ -222,7 +256,7 @@ __global__ __launch_bounds__(128) void dq_kernel(const BwdParams prm) {
     for (int ts = 0; ts < 4; ++ts)
 #pragma unroll
       for (int db = 0; db < DB; ++db)
-        dqacc[db] = mfma_f16(frag_cols<D, BF16>(kt, db, ts, lane), dsf[ts], dqacc[db]);          // dQ^T += K^T dS^T
+        dqacc[db] = mfma_f16(fkt[ts][db], dsf[ts], dqacc[db]);          // dQ^T += K^T dS^T
   }
 
   void* base = prm.out_f32 ? (void*)((float*)prm.dq + (int64_t)bh * prm.N * D) : (void*)((unsigned short*)prm.dq + (int64_t)bh * prm.N * D);
@@ -246,8 +280,10 @@ __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
   const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int ln = lane & 31, g = lane >> 5;
   const int nb = prm.nb;
-  const int n = blockIdx.x;                   // early columns of block-causal masks are the long ones
-  const int bh = blockIdx.y, b = bh / prm.H, h = bh % prm.H;
+  int bh, n;                                  // early columns of block-causal masks are the long ones
+  head_and_block(blockIdx.x, prm.B * prm.H, nb, bh, n);
+  if (n >= nb) return;
+  const int b = bh / prm.H, h = bh % prm.H;
   const int mh = (prm.Bm > 1 ? b : 0) * prm.Hm + (prm.Hm > 1 ? h : 0);
   const cint_ptr_t cp = (cint_ptr_t)(uintptr_t)(prm.col_ptr + (int64_t)mh * nb);
   const cint_ptr_t rows = (cint_ptr_t)(uintptr_t)prm.row_idx;
@@ -293,6 +329,16 @@ __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
     const float* st_lse = reinterpret_cast<const float*>(gt + C::TILE_BYTES);
     const float* st_dlt = st_lse + 64;
 
+    // operand fragments are read from LDS ahead of the block of MFMAs that consumes them
+    uintx4 fq[2][KS], fg[2][KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+#pragma unroll
+      for (int qb = 0; qb < 2; ++qb) {
+        fq[qb][s] = frag_rows<D>(qt, 32 * qb, s, ln, g);
+        fg[qb][s] = frag_rows<D>(gt, 32 * qb, s, ln, g);
+      }
+    __builtin_amdgcn_sched_barrier(0);
     floatx16 sacc[2], dpacc[2];
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) { sacc[qb] = zero16(); dpacc[qb] = zero16(); }
@@ -300,9 +346,20 @@ __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
     for (int s = 0; s < KS; ++s)
 #pragma unroll
       for (int qb = 0; qb < 2; ++qb) {
-        sacc[qb] = mfma_qk<BF16>(frag_rows<D>(qt, 32 * qb, s, ln, g), kfr[s], sacc[qb]);      // S = Q K^T
-        dpacc[qb] = mfma_qk<BF16>(frag_rows<D>(gt, 32 * qb, s, ln, g), vfr[s], dpacc[qb]);    // dP = dO V^T
+        sacc[qb] = mfma_qk<BF16>(fq[qb][s], kfr[s], sacc[qb]);      // S = Q K^T
+        dpacc[qb] = mfma_qk<BF16>(fg[qb][s], vfr[s], dpacc[qb]);    // dP = dO V^T
       }
+    __builtin_amdgcn_sched_barrier(0);
+    // dO^T and Q^T fragments of the second products, read under the exponentials below
+    uintx4 fgt[4][DB], fqt[4][DB];
+#pragma unroll
+    for (int ts = 0; ts < 4; ++ts)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        fgt[ts][db] = frag_cols<D, BF16>(gt, db, ts, lane);
+        fqt[ts][db] = frag_cols<D, BF16>(qt, db, ts, lane);
+      }
+    __builtin_amdgcn_sched_barrier(0);
     // rows of the results are queries: register i of block qb <-> query 32qb + 8(i/4) + 4g + i%4
     uintx4 pf[4], dsf[4];
 #pragma unroll
@@ -326,8 +383,8 @@ __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
     for (int ts = 0; ts < 4; ++ts)
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        dvacc[db] = mfma_f16(frag_cols<D, BF16>(gt, db, ts, lane), pf[ts], dvacc[db]);    // dV^T += dO^T P
-        dkacc[db] = mfma_f16(frag_cols<D, BF16>(qt, db, ts, lane), dsf[ts], dkacc[db]);   // dK^T += Q^T dS
+        dvacc[db] = mfma_f16(fgt[ts][db], pf[ts], dvacc[db]);    // dV^T += dO^T P
+        dkacc[db] = mfma_f16(fqt[ts][db], dsf[ts], dkacc[db]);   // dK^T += Q^T dS
       }
   }
 
@@ -368,8 +425,9 @@ static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
   const int BH = prm.B * prm.H;
   constexpr int RPB = 256 / (D / 8);
   hipLaunchKernelGGL((delta_kernel<D, BF16>), dim3((prm.N + RPB - 1) / RPB, BH), dim3(256), 0, st, prm);
-  hipLaunchKernelGGL((dq_kernel<D, BF16>), dim3(prm.nb, BH), dim3(128), C::LDS_BYTES, st, prm);
-  hipLaunchKernelGGL((dkdv_kernel<D, BF16>), dim3(prm.nb, BH), dim3(128), C::LDS_BYTES, st, prm);
+  const int grid = ((BH + 7) / 8) * 8 * prm.nb;   // heads in groups of 8, the last group padded
+  hipLaunchKernelGGL((dq_kernel<D, BF16>), dim3(grid), dim3(128), C::LDS_BYTES, st, prm);
+  hipLaunchKernelGGL((dkdv_kernel<D, BF16>), dim3(grid), dim3(128), C::LDS_BYTES, st, prm);
 }
 
 int launch_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
