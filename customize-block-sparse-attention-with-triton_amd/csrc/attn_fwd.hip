@@ -131,6 +131,7 @@ template <int D> struct FwdCfg {
   static constexpr int R = TILE_BYTES / 256;                // accumulator registers exchanged per round
   static constexpr int ROUNDS = D / R;
   static constexpr int QPW = (R / 4) / NW;                  // output quads per wavefront and round
+  static constexpr int SHORT_ROW = 6 * NW;                  // row blocks up to this many tiles may go to one wavefront
 };
 
 template <int D, bool BF16, bool ROWS>
@@ -401,33 +402,15 @@ void fwd_kernel(const FwdParams prm) {
     for (int i = threadIdx.x; i < t_hi - t_lo && i < C::COLS_CAP; i += NW * 64) lcols[i] = prm.col_idx[t_lo + i];
   };
 
-  if constexpr (ROWS) {
-    // ================= one wavefront per row block =================
-    // The workgroup owns the row blocks whose first kept tile lies in its range [g0, g1); they are
-    // handed out to the wavefronts through the LDS counter, and a wavefront runs a whole row block
-    // alone and writes its result directly: no merge, no partials.
-    int r_lo, r_hi;
-    {
-      int lo = -1, hi = nb;   // smallest r with rp[r] >= g0
-      while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (rp[mid] >= g0) hi = mid; else lo = mid; }
-      r_lo = hi;
-      lo = -1; hi = nb;       // smallest r with rp[r] >= g1
-      while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (rp[mid] >= g1) hi = mid; else lo = mid; }
-      r_hi = hi;
-      if (wg >= hs.Peff - 1) r_hi = nb;    // trailing row blocks without kept tiles
-      if (wg == 0) r_lo = 0;               // leading ones
-    }
-    const int t_lo = rp[r_lo];
-    stage_cols(t_lo, rp[r_hi]);
-    if (threadIdx.x == 0) *ctr = r_lo + 2 * NW;
-    __syncthreads();
-    auto col_of = [&](int t) { return t - t_lo < C::COLS_CAP ? lcols[t - t_lo] : (int)cols[t]; };
-    void* obase = out_base(prm, b, h);
+  // Whole row blocks [r_lo, r_hi), one wavefront each: handed out through the LDS counter *rctr
+  // (set to r_lo + 2 NW beforehand), written directly, nothing to merge.
+  void* obase = out_base(prm, b, h);
+  auto run_rows = [&](int r_lo, int r_hi, int* rctr, auto&& col_of) {
     int row = r_lo + w, row_next = r_lo + NW + w;     // the first two rounds are fixed
     int kdone = -1;                                    // tile whose K and V copies were issued ahead
     while (row < r_hi) {
       int drawn = 0;
-      if (lane == 0) drawn = atomicAdd(ctr, 1);       // the row block after next
+      if (lane == 0) drawn = atomicAdd(rctr, 1);       // the row block after next
       const int ta = rp[row], tb = rp[row + 1];
       // first tile of the next row block of this wavefront (prefetched under the last tile)
       const int tn = row_next < r_hi ? rp[row_next] : 0;
@@ -481,6 +464,30 @@ void fwd_kernel(const FwdParams prm) {
       row = row_next;
       row_next = __builtin_amdgcn_readfirstlane(drawn);
     }
+  };
+
+  if constexpr (ROWS) {
+    // ================= one wavefront per row block =================
+    // The workgroup owns the row blocks whose first kept tile lies in its range [g0, g1); they are
+    // handed out to the wavefronts through the LDS counter, and a wavefront runs a whole row block
+    // alone and writes its result directly: no merge, no partials.
+    int r_lo, r_hi;
+    {
+      int lo = -1, hi = nb;   // smallest r with rp[r] >= g0
+      while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (rp[mid] >= g0) hi = mid; else lo = mid; }
+      r_lo = hi;
+      lo = -1; hi = nb;       // smallest r with rp[r] >= g1
+      while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (rp[mid] >= g1) hi = mid; else lo = mid; }
+      r_hi = hi;
+      if (wg >= hs.Peff - 1) r_hi = nb;    // trailing row blocks without kept tiles
+      if (wg == 0) r_lo = 0;               // leading ones
+    }
+    const int t_lo = rp[r_lo];
+    stage_cols(t_lo, rp[r_hi]);
+    if (threadIdx.x == 0) *ctr = r_lo + 2 * NW;
+    __syncthreads();
+    auto col_of = [&](int t) { return t - t_lo < C::COLS_CAP ? lcols[t - t_lo] : (int)cols[t]; };
+    run_rows(r_lo, r_hi, ctr, col_of);
   } else {
     // ================= all wavefronts on one row block at a time =================
     // Tiles of the range are handed out to the wavefronts dynamically (the LDS counter), because
@@ -498,16 +505,49 @@ void fwd_kernel(const FwdParams prm) {
       r = lo;
     }
     stage_cols(g0, g1);
-    if (threadIdx.x == 0) *ctr = g0 + 2 * NW;
+    if (threadIdx.x == 0) { ctr[0] = g0 + 2 * NW; ctr[3] = 0; }
     __syncthreads();
     auto col_of = [&](int t) { return t - g0 < C::COLS_CAP ? lcols[t - g0] : (int)cols[t]; };
     int cur = g0 + w, nxt = g0 + NW + w;      // the first two rounds are fixed
     int cb_nxt = nxt < g1 ? __builtin_amdgcn_readfirstlane(col_of(nxt)) : 0;   // column block of tile nxt
     int kdone = -1, vdone = -1;
     int t = g0;
+    const int32_t* rpg = prm.row_ptr + (int64_t)mh * nb;
     while (t < g1) {
       const int row_s = rp[r], row_e = rp[r + 1];
       if (row_e <= t) { ++r; continue; }          // row block without kept tiles in the range
+      // A run of short row blocks that lie completely inside the range is not worth a merge per
+      // row block: such a run is done one row block per wavefront.  Every wavefront looks at the
+      // next 64 row blocks (one per lane) and comes to the same decision.
+      if (t == row_s && row_e <= g1 && row_e - row_s <= C::SHORT_ROW) {
+        const int idx = r + lane;
+        const int rs_i = idx < nb ? rpg[idx] : 0, re_i = idx < nb ? rpg[idx + 1] : 0x7fffffff;
+        const bool ok_i = idx < nb && re_i <= g1 && re_i - rs_i <= C::SHORT_ROW;
+        const unsigned long long okm = __ballot(ok_i);
+        const int cnt = ~okm == 0ull ? 64 : __builtin_ctzll(~okm);        // leading run of short inner row blocks
+        const bool in_run = lane < cnt;
+        const int bn = __builtin_popcountll(__ballot(in_run && re_i > rs_i));   // ... with kept tiles
+        int maxlen = in_run ? re_i - rs_i : 0;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) { const int o = __shfl_xor(maxlen, off); maxlen = o > maxlen ? o : maxlen; }
+        maxlen = __builtin_amdgcn_readfirstlane(maxlen);
+        // worth it when the run keeps the wavefronts busy, or when its row blocks are short
+        // against the cost of a merge (about three tiles per wavefront)
+        const bool batch = bn >= NW || (bn == 3) || (bn == 2 && maxlen < 3 * NW) || (bn == 1 && maxlen < NW);
+        if (batch) {
+          const int r2 = r + cnt, t2 = __builtin_amdgcn_readfirstlane(__shfl(re_i, cnt - 1));
+          wait_vm<0>();                 // prefetches of the tile hand-out below are abandoned
+          __syncthreads();              // everybody has left the previous run and the previous merge
+          if (threadIdx.x == 0) { ctr[2] = r + 2 * NW; ctr[0] = t2 + 2 * NW; }
+          __syncthreads();
+          run_rows(r, r2, ctr + 2, col_of);
+          cur = t2 + w; nxt = t2 + NW + w;
+          cb_nxt = nxt < g1 ? __builtin_amdgcn_readfirstlane(col_of(nxt)) : 0;
+          kdone = -1; vdone = -1;
+          t = t2; r = r2;
+          continue;
+        }
+      }
       const int seg_a = t, seg_b = row_e < g1 ? row_e : g1;
       const bool mine = cur < seg_b;      // this wavefront processes at least one tile of the row block
       reset_acc();
@@ -558,8 +598,12 @@ void fwd_kernel(const FwdParams prm) {
         float wgt[NW][2];   // weight of wavefront p's partial for this lane's query of block qb
         float M[2], L[2];
         float keep[C::ROUNDS][C::QPW][4];   // this wavefront's share of the merged accumulator (pull)
-        float* slot = prm.ws + ((int64_t)bh * prm.W + wg) * partial_floats(D);
-        void* obase = out_base(prm, b, h);
+        // A zero the compiler cannot see through (ctr[3] stays 0): the per-lane addresses into the
+        // workspace do not change from row block to row block and would otherwise be computed
+        // once, up front, and occupy registers throughout the tile loops.
+        typedef volatile int __attribute__((address_space(3)))* lds_vint_ptr_t;
+        const int zero = *(lds_vint_ptr_t)(lds_ptr_t)(ctr + 3);
+        float* slot = prm.ws + ((int64_t)bh * prm.W + wg) * partial_floats(D) + zero;
 #pragma unroll
         for (int rd = 0; rd < C::ROUNDS; ++rd) {
           {
@@ -649,26 +693,39 @@ void fwd_kernel(const FwdParams prm) {
               if (__builtin_amdgcn_s_memrealtime() - t_start > 20000000ll) { ok = false; break; }
               __builtin_amdgcn_s_sleep(4);
             }
-            const float* sp = prm.ws + ((int64_t)bh * prm.W + p) * partial_floats(D);
+            const float* sp = prm.ws + ((int64_t)bh * prm.W + p) * partial_floats(D) + zero;
+            // all loads of the part are issued before the first one is waited for (a round trip
+            // to the point of coherence costs about a microsecond)
+            float mp[2], lp[2], dat[C::ROUNDS][C::QPW][4];
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb) {
+              mp[qb] = coherent_load(sp + 64 * D + qb * 32 + ln);
+              lp[qb] = coherent_load(sp + 64 * D + 64 + qb * 32 + ln);
+            }
+#pragma unroll
+            for (int rd = 0; rd < C::ROUNDS; ++rd)
+#pragma unroll
+              for (int tq = 0; tq < C::QPW; ++tq)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                  dat[rd][tq][e] = coherent_load(sp + (rd * C::R + 4 * (w * C::QPW + tq) + e) * 64 + lane);
+            __builtin_amdgcn_sched_barrier(0);
             float sc_own[2], sc_p[2];
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb) {
-              const float mp = coherent_load(sp + 64 * D + qb * 32 + ln), lp = coherent_load(sp + 64 * D + 64 + qb * 32 + ln);
-              const float mn = fmaxf(M[qb], mp);
+              const float mn = fmaxf(M[qb], mp[qb]);
               sc_own[qb] = __builtin_amdgcn_exp2f(M[qb] - mn);
-              sc_p[qb] = __builtin_amdgcn_exp2f(mp - mn);
-              L[qb] = L[qb] * sc_own[qb] + lp * sc_p[qb];
+              sc_p[qb] = __builtin_amdgcn_exp2f(mp[qb] - mn);
+              L[qb] = L[qb] * sc_own[qb] + lp[qb] * sc_p[qb];
               M[qb] = mn;
             }
 #pragma unroll
             for (int rd = 0; rd < C::ROUNDS; ++rd)
 #pragma unroll
               for (int tq = 0; tq < C::QPW; ++tq) {
-                const int idx0 = rd * C::R + 4 * (w * C::QPW + tq);
-                const int qb = (idx0 / 16) & 1;
+                const int qb = ((rd * C::R + 4 * (w * C::QPW + tq)) / 16) & 1;
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                  keep[rd][tq][e] = keep[rd][tq][e] * sc_own[qb] + sc_p[qb] * coherent_load(sp + (idx0 + e) * 64 + lane);
+                for (int e = 0; e < 4; ++e) keep[rd][tq][e] = keep[rd][tq][e] * sc_own[qb] + sc_p[qb] * dat[rd][tq][e];
               }
           }
           const float bad = ok ? 0.f : __builtin_nanf("");

@@ -97,6 +97,30 @@ def test_row_block_per_wavefront_several_workgroups_per_head(dev):
     run_case(dev, 2, 32, 2048, 64, torch.bfloat16, m2, 6, out_fp32=True)
 
 
+@pytest.mark.parametrize("D,dtype", [(64, torch.float16), (128, torch.bfloat16)])
+def test_short_and_long_row_blocks_mixed(dev, D, dtype):
+    """Runs of short row blocks inside a workgroup's range go one row block per wavefront, long
+    ones are shared by the wavefronts: block-causal masks (lengths 1..nb), alternating short / long /
+    empty row blocks, and a mask whose row blocks all hold one or two tiles."""
+    nb = 48
+    run_case(dev, 1, 2, nb * 64, D, dtype, causal_block_mask(1, 1, nb, 0.6, 3), 41, out_fp32=True)
+    g = torch.Generator().manual_seed(9)
+    m = torch.zeros(1, 2, nb, nb, dtype=torch.bool)
+    for r in range(nb):
+        kind = r % 5
+        if kind in (0, 1, 3):
+            m[0, :, r, torch.randperm(nb, generator=g)[:1 + r % 3]] = True      # 1..3 tiles
+        elif kind == 2:
+            m[0, 0, r, :] = True                                                   # long
+            m[0, 1, r, torch.randperm(nb, generator=g)[:30]] = True
+        # kind 4: empty
+    run_case(dev, 1, 2, nb * 64, D, dtype, m, 42, out_fp32=True)
+    m2 = torch.zeros(2, 3, nb, nb, dtype=torch.bool)
+    idx = torch.randint(0, nb, (2, 3, nb, 2), generator=g)
+    m2.scatter_(3, idx, True)
+    run_case(dev, 2, 3, nb * 64, D, dtype, m2, 43, out_fp32=True)
+
+
 def test_workspace_contents_do_not_matter(dev):
     """Row blocks shared between workgroups are merged by whichever workgroup arrives last, counted
     in the workspace: stale or random workspace contents, and repeated runs on the same workspace,
