@@ -406,15 +406,18 @@ void fwd_kernel(const FwdParams prm) {
   // (set to r_lo + 2 NW beforehand), written directly, nothing to merge.
   void* obase = out_base(prm, b, h);
   auto run_rows = [&](int r_lo, int r_hi, int* rctr, auto&& col_of) {
-    int row = r_lo + w, row_next = r_lo + NW + w;     // the first two rounds are fixed
+    // Tickets r_lo, r_lo + 1, ... stand for the row blocks r_hi - 1, r_hi - 2, ...: with block-causal
+    // masks the late row blocks are the long ones, and the long ones should not come last.
+    int tick = r_lo + w, tick_next = r_lo + NW + w;   // the first two rounds are fixed
     int kdone = -1;                                    // tile whose K and V copies were issued ahead
-    while (row < r_hi) {
+    while (tick < r_hi) {
       int drawn = 0;
       if (lane == 0) drawn = atomicAdd(rctr, 1);       // the row block after next
+      const int row = r_lo + r_hi - 1 - tick, row_next = r_lo + r_hi - 1 - tick_next;
       const int ta = rp[row], tb = rp[row + 1];
       // first tile of the next row block of this wavefront (prefetched under the last tile)
-      const int tn = row_next < r_hi ? rp[row_next] : 0;
-      const bool next_has = row_next < r_hi && rp[row_next + 1] > tn;
+      const int tn = tick_next < r_hi ? rp[row_next] : 0;
+      const bool next_has = tick_next < r_hi && rp[row_next + 1] > tn;
       if (ta < tb) {
         if (kdone != ta) {
           const int cb = __builtin_amdgcn_readfirstlane(col_of(ta));
@@ -461,8 +464,8 @@ void fwd_kernel(const FwdParams prm) {
           if (prm.lse != nullptr && g == 0) prm.lse[((int64_t)bh * prm.N) + qrow] = -INFINITY;
         }
       }
-      row = row_next;
-      row_next = __builtin_amdgcn_readfirstlane(drawn);
+      tick = tick_next;
+      tick_next = __builtin_amdgcn_readfirstlane(drawn);
     }
   };
 
