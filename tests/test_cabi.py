@@ -68,6 +68,17 @@ def test_argument_validation_without_gpu():
     assert l.bsattn_reorder(P, P, 1, 1, 2, 2, 2, 4, 2, None, None, None) == -1
 
 
+def test_mfma_rate_probe_validation_without_gpu():
+    from fa2_custom_mask import _ext
+    l = _ext.lib()
+    P = ctypes.c_void_p(4096)
+    assert l.bsattn_mfma_rate_probe(None, 16, P, None, None) == -1      # BSATTN_ERR_NULL
+    assert l.bsattn_mfma_rate_probe(P, 16, None, None, None) == -1
+    assert l.bsattn_mfma_rate_probe(P, 0, P, None, None) == -8          # BSATTN_ERR_RANGE
+    assert l.bsattn_mfma_rate_probe(P, 1 << 21, P, None, None) == -8
+    assert l.bsattn_mfma_rate_probe(ctypes.c_void_p(4100), 16, P, None, None) == -5   # BSATTN_ERR_STRIDE (alignment)
+
+
 def test_python_wrapper_rejects_bad_input_without_gpu():
     import torch
     import fa2_custom_mask as fm

@@ -85,3 +85,21 @@ def test_c5_fwd_bwd_bf16_d128(dev):
     for a, b_ in ((o16, o), (dq16, dq), (dk16, dk), (dv16, dv)):
         assert a.dtype == torch.bfloat16
         assert errors(a, b_)[1] <= 3e-3                           # the same values up to bf16 rounding
+
+
+def test_mfma_rate_probe_runs(dev):
+    """The measurement aid launches, reports the FLOPs of the launch and leaves finite sums."""
+    import ctypes
+    from fa2_custom_mask import _ext
+    lib = _ext.lib()
+    ops = torch.ones(4096, dtype=torch.float16, device=dev)
+    sink = torch.full((512,), float("nan"), dtype=torch.float32, device=dev)
+    flops = ctypes.c_double()
+    st = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    rc = lib.bsattn_mfma_rate_probe(ops.data_ptr(), 4, sink.data_ptr(), ctypes.byref(flops), st)
+    assert rc == 0
+    torch.cuda.synchronize()
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    assert flops.value == cus * 8 * 4 * 8 * 2 * 32 * 32 * 16
+    # every accumulator element is 4 iterations x 2 MFMAs per chain x 16 ones = 128; 64 elements per lane
+    assert torch.all(sink == 128.0 * 64)
