@@ -9,7 +9,7 @@ import ctypes
 import torch
 
 from . import _ext
-from .utils import TILE, block_mask_to_lists, to_block_mask, _check_mask
+from .utils import TILE, block_mask_to_lists, mask_to_lists, to_block_mask, _check_mask
 
 
 def build_groups_from_block_mask(mask):
@@ -46,12 +46,23 @@ def _check_qkv(q, k, v, mask):
     if N % TILE != 0:
         raise ValueError("sequence length must be a multiple of 64")
     if mask is None:
-        raise ValueError("mask=None is not supported (the reference has no dense path either: "
-                         "`groups` is unbound at fa2_custom_mask.py:69)")
+        return B, H, N, D
     _check_mask(mask)
     if mask.shape[0] not in (1, B) or mask.shape[1] not in (1, H):
         raise ValueError("mask batch/head sizes must be 1 or match q")
     return B, H, N, D
+
+
+_all_true = {}
+
+
+def _dense_mask(device, nb):
+    """mask=None means plain dense attention (the reference advertises the default but crashes on
+    it: `groups` is unbound at fa2_custom_mask.py:69): one all-true block mask shared by all heads."""
+    key = (device, nb)
+    if key not in _all_true:
+        _all_true[key] = torch.ones((1, 1, nb, nb), dtype=torch.bool, device=device)
+    return _all_true[key]
 
 
 def _forward(q, k, v, lists, sm_scale, out_dtype, want_lse):
@@ -125,11 +136,12 @@ class _attention(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, mask=None, sm_scale=1.3, out_fp32=False, return_lse=False):
         B, H, N, D = _check_qkv(q, k, v, mask)
-        block = to_block_mask(mask, N)
-        lists = block_mask_to_lists(block)                                   # :48
+        if mask is None:
+            mask = _dense_mask(q.device, N // TILE)
+        lists = mask_to_lists(mask, N)                                       # :48
         out_dtype = torch.float32 if out_fp32 else q.dtype
         o, lse = _forward(q, k, v, lists, sm_scale, out_dtype, True)
-        ctx.save_for_backward(q, k, v, o, lse, block)                        # :89
+        ctx.save_for_backward(q, k, v, o, lse, mask)                         # :89
         ctx.lists = lists
         ctx.sm_scale = sm_scale
         ctx.out_dtype = out_dtype
@@ -141,8 +153,8 @@ class _attention(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, do, *unused):
-        q, k, v, o, lse, block = ctx.saved_tensors
-        lists_t = block_mask_to_lists(block, transpose=True)
+        q, k, v, o, lse, mask = ctx.saved_tensors
+        lists_t = mask_to_lists(mask, q.shape[2], transpose=True)
         o_in = o if o.dtype == q.dtype else o.to(q.dtype)
         do_in = do if do.dtype == q.dtype else do.to(q.dtype)
         # autograd hands gradients back in the dtype of q, k, v
@@ -153,7 +165,8 @@ class _attention(torch.autograd.Function):
 def flash_attention_custom_mask(q, k, v, mask=None, sm_scale=1.3):
     """Drop-in for the reference's `flash_attention_custom_mask = _attention.apply`
     (fa2_custom_mask.py:157): q,k,v [B,H,N,D] fp16/bf16 on the GPU, mask bool
-    [B|1,H|1,N/64,N/64] (or elementwise [B|1,H|1,N,N]), returns o like q."""
+    [B|1,H|1,N/64,N/64] (or elementwise [B|1,H|1,N,N]; None = dense attention), returns o like
+    q.  The kept-tile lists of a mask tensor are cached until the tensor is modified."""
     return _attention.apply(q, k, v, mask, sm_scale)
 
 
@@ -168,9 +181,10 @@ def attention_forward_backward(q, k, v, mask, sm_scale, do, out_fp32=False):
     """Non-autograd entry: (o, lse, dq, dk, dv) in one call; with out_fp32 all five results
     are fp32 (autograd itself can only hand back gradients in the dtype of q)."""
     B, H, N, D = _check_qkv(q, k, v, mask)
-    block = to_block_mask(mask, N)
-    lists = block_mask_to_lists(block)
-    lists_t = block_mask_to_lists(block, transpose=True)
+    if mask is None:
+        mask = _dense_mask(q.device, N // TILE)
+    lists = mask_to_lists(mask, N)
+    lists_t = mask_to_lists(mask, N, transpose=True)
     out_dtype = torch.float32 if out_fp32 else q.dtype
     o, lse = _forward(q, k, v, lists, sm_scale, out_dtype, True)
     o_in = o if o.dtype == q.dtype else o.to(q.dtype)

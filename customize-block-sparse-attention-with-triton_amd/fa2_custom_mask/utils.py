@@ -3,6 +3,7 @@
 `is_hip` / `keep` keep the names exported by the reference (fa2_custom_mask/utils.py:3-14).
 """
 import ctypes
+import weakref
 
 import torch
 
@@ -98,3 +99,41 @@ def to_block_mask(mask, N):
         return reduce_dense_mask(mask)
     raise ValueError("mask shape %s matches neither [.., %d, %d] nor [.., %d, %d]"
                      % (tuple(mask.shape), nb, nb, N, N))
+
+
+class _ListsCache:
+    """Kept-tile lists of the most recently used masks.  A static mask (the usual case: one mask
+    for every layer and step) is indexed once instead of once per call.  An entry is only used
+    for the very tensor object it was built from, and only while that tensor has not been
+    written to (autograd's version counter)."""
+
+    def __init__(self, capacity=8):
+        self.capacity = capacity
+        self._entries = []     # (weakref to mask, version, N, transpose, lists), most recent last
+
+    def get(self, mask, N, transpose):
+        for i, (ref, ver, n, tr, lists) in enumerate(self._entries):
+            if ref() is mask and ver == mask._version and n == N and tr == transpose:
+                self._entries.append(self._entries.pop(i))
+                return lists
+        return None
+
+    def put(self, mask, N, transpose, lists):
+        self._entries = [e for e in self._entries if e[0]() is not None]
+        self._entries.append((weakref.ref(mask), mask._version, N, transpose, lists))
+        del self._entries[:-self.capacity]
+
+    def clear(self):
+        self._entries = []
+
+
+lists_cache = _ListsCache()
+
+
+def mask_to_lists(mask, N, transpose=False):
+    """TileLists of a block or elementwise mask for sequence length N, through the cache."""
+    lists = lists_cache.get(mask, N, transpose)
+    if lists is None:
+        lists = block_mask_to_lists(to_block_mask(mask, N), transpose=transpose)
+        lists_cache.put(mask, N, transpose, lists)
+    return lists

@@ -121,6 +121,47 @@ def test_short_and_long_row_blocks_mixed(dev, D, dtype):
     run_case(dev, 2, 3, nb * 64, D, dtype, m2, 43, out_fp32=True)
 
 
+def test_mask_none_is_dense_attention(dev):
+    """mask=None (the default the reference advertises, fa2_custom_mask.py:43) = dense attention:
+    against torch's scaled_dot_product_attention in fp32, forward and backward."""
+    import fa2_custom_mask as fm
+    q, k, v, do = [x.to(dev) for x in make_qkv(2, 2, 512, 64, torch.float16, 91, n=4)]
+    qr, kr, vr = [x.float().requires_grad_(True) for x in (q, k, v)]
+    ref = torch.nn.functional.scaled_dot_product_attention(qr, kr, vr, scale=0.125)
+    ref.backward(do.float())
+    qg, kg, vg = [x.clone().requires_grad_(True) for x in (q, k, v)]
+    o = fm.flash_attention_custom_mask(qg, kg, vg, None, 0.125)
+    o.backward(do)
+    assert errors(o, ref.detach().cpu().numpy())[0] <= 2e-2
+    for got, want in ((qg.grad, qr.grad), (kg.grad, kr.grad), (vg.grad, vr.grad)):
+        assert errors(got, want.cpu().numpy())[0] <= 2e-2
+
+
+def test_lists_cache_follows_the_mask(dev):
+    """The kept-tile lists of a mask tensor are reused while the tensor is unchanged and rebuilt
+    after an in-place change or for another tensor."""
+    import fa2_custom_mask as fm
+    from fa2_custom_mask import utils
+    q, k, v = [x.to(dev) for x in make_qkv(1, 1, 512, 64, torch.float16, 92)]
+    m = uniform_block_mask(1, 1, 8, 0.5, 93)
+    md = m.to(dev)
+    utils.lists_cache.clear()
+    o1 = fm.flash_attention_custom_mask(q, k, v, md, 0.125)
+    first = utils.lists_cache.get(md, 512, False)
+    assert first is not None
+    o2 = fm.flash_attention_custom_mask(q, k, v, md, 0.125)
+    assert utils.lists_cache.get(md, 512, False) is first and same_up_to_rounding(o1, o2)
+    m[0, 0, 2, :] = ~m[0, 0, 2, :]
+    m[0, 0, 2, 2] = True
+    md.copy_(m)                                   # in place: same tensor object, new contents
+    assert utils.lists_cache.get(md, 512, False) is None
+    o3 = fm.flash_attention_custom_mask(q, k, v, md, 0.125)
+    o_ref = orc.naive_attention(f32(q), f32(k), f32(v), m.numpy(), 0.125)
+    assert errors(o3, o_ref)[0] <= 2e-2
+    md2 = m.to(dev)                               # equal contents, different tensor: not shared
+    assert utils.lists_cache.get(md2, 512, False) is None
+
+
 def test_workspace_contents_do_not_matter(dev):
     """Row blocks shared between workgroups are merged by whichever workgroup arrives last, counted
     in the workspace: stale or random workspace contents, and repeated runs on the same workspace,
