@@ -54,6 +54,18 @@ int bsattn_block_mask_to_lists(const uint8_t* block, int Bm, int Hm, int nb, int
                                     (int32_t*)workspace, (hipStream_t)stream);
 }
 
+int bsattn_pack_mask_tiles(const uint8_t* dense, int Bm, int Hm, int N, int64_t sb, int64_t sh, int64_t sm,
+                           int64_t sn, const int32_t* row_ptr, const int32_t* col_idx, uint8_t* tile_partial,
+                           uint64_t* tile_bits, void* stream) {
+  if (dense == nullptr || row_ptr == nullptr || col_idx == nullptr || tile_partial == nullptr || tile_bits == nullptr)
+    return BSATTN_ERR_NULL;
+  if (Bm <= 0 || Hm <= 0 || N <= 0 || N % BSATTN_TILE != 0) return BSATTN_ERR_SHAPE;
+  if ((int64_t)Bm * Hm > 65535) return BSATTN_ERR_RANGE;
+  if (sn == 1 && ((sm % 4) != 0 || (sb % 4) != 0 || (sh % 4) != 0 || ((uintptr_t)dense & 3) != 0)) return BSATTN_ERR_STRIDE;
+  return launch_pack_tiles(dense, Bm, Hm, N / BSATTN_TILE, sb, sh, sm, sn, row_ptr, col_idx, tile_partial,
+                           (unsigned long long*)tile_bits, (hipStream_t)stream);
+}
+
 static int check_attn(int Bm, int Hm, int B, int H, int N, int D, int dtype, int out_dtype) {
   if (B <= 0 || H <= 0 || N <= 0 || N % BSATTN_TILE != 0) return BSATTN_ERR_SHAPE;
   if (!((Bm == 1 || Bm == B) && (Hm == 1 || Hm == H))) return BSATTN_ERR_SHAPE;

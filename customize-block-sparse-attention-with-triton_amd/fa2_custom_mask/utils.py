@@ -89,6 +89,31 @@ def block_mask_to_lists(block, transpose=False, want_groups=False):
     return TileLists(row_ptr, col_idx, groups, counts, Bm, Hm, nb)
 
 
+def pack_mask_tiles(mask, lists, transpose=False):
+    """Elementwise mask [Bm,Hm,N,N] + the TileLists of its reduced form -> (tile_partial uint8
+    [cap], tile_bits int64 [cap, 64]) with one slot per kept tile: is the tile only partly set,
+    and its 64 x 64 bools as 64 words (word r, bit c = element (r, c) of the tile; with
+    transpose=True, matching transposed lists, element (c, r))."""
+    _check_mask(mask)
+    Bm, Hm, N, N2 = mask.shape
+    if N != N2 or N % TILE != 0 or N // TILE != lists.nb or (Bm, Hm) != (lists.Bm, lists.Hm):
+        raise ValueError("mask and lists do not belong together")
+    sb, sh, sm, sn = mask.stride()
+    if min(sm, sn) != 1 or any(s % 4 for s in (sb, sh, max(sm, sn))) or mask.data_ptr() % 4:
+        mask = mask.contiguous()
+        sb, sh, sm, sn = mask.stride()
+    if transpose:
+        sm, sn = sn, sm
+    cap = Bm * Hm * lists.nb * lists.nb
+    partial = torch.empty(cap, dtype=torch.uint8, device=mask.device)
+    bits = torch.empty((cap, 64), dtype=torch.int64, device=mask.device)
+    rc = _ext.lib().bsattn_pack_mask_tiles(mask.data_ptr(), Bm, Hm, N, sb, sh, sm, sn, lists.row_ptr.data_ptr(),
+                                           lists.col_idx.data_ptr(), partial.data_ptr(), bits.data_ptr(),
+                                           _ext.current_stream(mask.device))
+    _ext.check(rc, "bsattn_pack_mask_tiles")
+    return partial, bits
+
+
 def to_block_mask(mask, N):
     """Accepts the reference's block form [.,.,N/64,N/64] or an elementwise [.,.,N,N] mask."""
     _check_mask(mask)

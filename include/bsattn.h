@@ -84,6 +84,22 @@ int bsattn_block_mask_to_lists(const uint8_t* block, int Bm, int Hm, int nb,
                                void* stream);
 
 /* ------------------------------------------------------------------------------------
+ * Elementwise masks (exact semantics inside partly set tiles: the naive masked_fill(-inf)
+ * of kernel-test.py:38, which the reference's dead elementwise loop fa2_fwd.py:67-73 and
+ * its backward fa2_bwd.py:59-62,119-123 intend).  For every entry t of the kept-tile lists
+ * of the reduced mask: tile_partial[t] = 1 if the tile is only partly set, and
+ * tile_bits[64 t + r] = the 64 bools of row r of the tile (bit c = column c).
+ * dense: bool bytes [Bm,Hm,N,N] with element strides sb, sh, sm (rows), sn (columns);
+ * row_ptr/col_idx: lists of the reduced mask as made by bsattn_block_mask_to_lists.
+ * Passing the lists of the transposed block mask together with sm and sn swapped gives
+ * the per-key words the dK/dV pass uses.  tile_partial: nb*nb*Bm*Hm bytes capacity,
+ * tile_bits: 64 times as many 64-bit words.  sn == 1 needs 4-byte aligned rows.
+ * ---------------------------------------------------------------------------------- */
+int bsattn_pack_mask_tiles(const uint8_t* dense, int Bm, int Hm, int N, int64_t sb, int64_t sh,
+                           int64_t sm, int64_t sn, const int32_t* row_ptr, const int32_t* col_idx,
+                           uint8_t* tile_partial, uint64_t* tile_bits, void* stream);
+
+/* ------------------------------------------------------------------------------------
  * Forward.  Replaces the launch of _attn_fwd (fa2_custom_mask/fa2_fwd.py:108-206) from
  * _attention.forward (fa2_custom_mask/fa2_custom_mask.py:69-87).
  * ---------------------------------------------------------------------------------- */

@@ -105,12 +105,45 @@ def _bcast_mask(block_mask, B, H):
     return np.broadcast_to(block_mask, (B, H) + block_mask.shape[2:])
 
 
+def _keep_rows(mask_bh, N, r0, r1):
+    """Elementwise keep matrix of query rows [r0, r1): the mask of one head is either a block
+    mask [N/64, N/64] (expanded as kernel-test.py:18) or already elementwise [N, N]."""
+    if mask_bh.shape[-1] == N and N != N // TILE:
+        return mask_bh[r0:r1]
+    return np.repeat(np.repeat(mask_bh[r0 // TILE:r1 // TILE], TILE, 0), TILE, 1)
+
+
+def pack_mask_tiles(dense, transpose=False):
+    """Data format of the elementwise-mask path (no counterpart in the reference): for every
+    kept tile of the reduced mask, in list order (row lists, or column lists with
+    transpose=True): partial flag (tile not completely set) and 64 words, word r bit c =
+    element (r, c) of the tile (element (c, r) with transpose=True).  Plain loops."""
+    dense = np.asarray(dense, dtype=bool)
+    Bm, Hm, N, _ = dense.shape
+    nb = N // TILE
+    partial, words = [], []
+    for b in range(Bm):
+        for h in range(Hm):
+            for a in range(nb):
+                for c in range(nb):
+                    rb, cb = (c, a) if transpose else (a, c)
+                    t = dense[b, h, rb * TILE:(rb + 1) * TILE, cb * TILE:(cb + 1) * TILE]
+                    if not t.any():
+                        continue
+                    if transpose:
+                        t = t.T
+                    partial.append(0 if t.all() else 1)
+                    words.append([sum(int(t[r, cc]) << cc for cc in range(TILE)) for r in range(TILE)])
+    return np.array(partial, dtype=np.uint8), np.array(words, dtype=np.uint64).reshape(-1, TILE)
+
+
 def naive_attention(q, k, v, block_mask, sm_scale, dtype=np.float32, row_chunk=2048,
                     return_lse=False):
     """kernel-test.py:37-40: attn = q@k^T*sm_scale; masked_fill(~mask,-inf); softmax; attn@v.
 
     q,k,v: [B,H,N,D] arrays (any float dtype; upcast to `dtype`).  block_mask:
-    [B|1, H|1, N/64, N/64] bool, expanded as kernel-test.py:18.  Query rows are processed
+    [B|1, H|1, N/64, N/64] bool, expanded as kernel-test.py:18, or an elementwise
+    [B|1, H|1, N, N] bool mask used as it is.  Query rows are processed
     in chunks, which is exact for a row-wise softmax.  Rows without any kept key give
     O = 0 and lse = -inf here (the reference's naive path gives NaN, its kernel leaves
     the row unwritten: fa2_custom_mask.py:29-30,59).
@@ -127,7 +160,7 @@ def naive_attention(q, k, v, block_mask, sm_scale, dtype=np.float32, row_chunk=2
             for r0 in range(0, N, row_chunk):
                 r1 = min(N, r0 + row_chunk)
                 s = (q[b, h, r0:r1] @ kt) * dtype(sm_scale)                    # :37
-                keep = np.repeat(np.repeat(bm[b, h, r0 // TILE:r1 // TILE], TILE, 0), TILE, 1)
+                keep = _keep_rows(bm[b, h], N, r0, r1)
                 s = np.where(keep, s, dtype(-np.inf))                          # :38
                 mx = s.max(axis=1, keepdims=True)
                 mx_safe = np.where(np.isfinite(mx), mx, dtype(0))
@@ -215,7 +248,7 @@ def attention_backward(q, k, v, block_mask, sm_scale, do, dtype=np.float32):
     delta = np.zeros((B, H, N), dtype=dtype)
     for b in range(B):
         for h in range(H):
-            keep = expand_block_mask(bm[b, h])
+            keep = _keep_rows(bm[b, h], N, 0, N)
             s = (q[b, h] @ k[b, h].T) * dtype(sm_scale)
             s = np.where(keep, s, dtype(-np.inf))
             mx = s.max(axis=1, keepdims=True)

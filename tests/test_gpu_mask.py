@@ -89,3 +89,29 @@ def test_dense_mask_partial_tiles(dev):
     red = fm.reduce_dense_mask(dense.to(dev)).cpu().numpy()
     assert np.array_equal(red, orc.reduce_dense_mask(dense.numpy()))
     assert red.sum() == len(pts)          # (0,0) and (63,63) share a tile
+
+
+@pytest.mark.parametrize("transpose", [False, True])
+def test_pack_mask_tiles_bit_exact(dev, transpose):
+    """Packed 64 x 64 tile words and partial flags of elementwise masks: bit-exact against the
+    oracle, for both list orientations, a shared (broadcast) mask and a non-contiguous view."""
+    import fa2_custom_mask as fm
+    from fa2_custom_mask import utils
+    g = torch.Generator().manual_seed(17)
+    for shape, p in (((1, 1, 256, 256), 0.5), ((2, 3, 192, 192), 0.05), ((1, 2, 320, 320), 0.9)):
+        dense = torch.rand(shape, generator=g) < p
+        dense[0, 0, :64, :64] = True
+        dense[0, -1, 64:128, :] = False
+        variants = [dense.to(dev)]
+        big = torch.zeros(shape[:3] + (shape[3] + 64,), dtype=torch.bool)
+        big[..., :shape[3]] = dense
+        variants.append(big.to(dev)[..., :shape[3]])                 # padded rows: not contiguous
+        for md in variants:
+            block = fm.reduce_dense_mask(md)
+            lists = fm.block_mask_to_lists(block, transpose=transpose)
+            partial, bits = utils.pack_mask_tiles(md, lists, transpose=transpose)
+            T = int(lists.counts[1])
+            p_ref, w_ref = orc.pack_mask_tiles(dense.numpy(), transpose)
+            assert T == len(p_ref)
+            assert np.array_equal(partial[:T].cpu().numpy(), p_ref)
+            assert np.array_equal(bits[:T].cpu().numpy().view(np.uint64), w_ref)

@@ -145,3 +145,34 @@ def test_backward_finite_differences():
             args_p[which] = ap; args_m[which] = am
             fd = (loss(*args_p) - loss(*args_m)) / (2 * eps)
             assert abs(fd - grad[idx]) < 1e-6 * max(1.0, abs(fd))
+
+
+def test_elementwise_mask_matches_sdpa_bool_mask():
+    """An arbitrary elementwise mask (every row keeps at least one key) against torch's
+    scaled_dot_product_attention with a boolean attn_mask, forward and gradients."""
+    g = torch.Generator().manual_seed(5)
+    B, H, N, D = 1, 2, 128, 16
+    q, k, v, do = [torch.randn(B, H, N, D, generator=g, dtype=torch.float64) for _ in range(4)]
+    m = torch.rand(1, H, N, N, generator=g) < 0.3
+    m |= torch.eye(N, dtype=torch.bool)
+    m[0, 0, 64:, :64] = False                     # an empty tile
+    m[0, 1, :64, 64:] = True                      # a full tile
+    qr, kr, vr = [x.clone().requires_grad_(True) for x in (q, k, v)]
+    ref = torch.nn.functional.scaled_dot_product_attention(qr, kr, vr, attn_mask=m, scale=0.25)
+    ref.backward(do)
+    o, lse = orc.naive_attention(q.numpy(), k.numpy(), v.numpy(), m.numpy(), 0.25, dtype=np.float64, return_lse=True)
+    assert np.abs(o - ref.detach().numpy()).max() < 1e-12
+    s = (q @ k.transpose(-1, -2) * 0.25).masked_fill(~m, float("-inf"))
+    assert np.abs(lse - torch.logsumexp(s, -1).numpy()).max() < 1e-12
+    dq, dk, dv, _ = orc.attention_backward(q.numpy(), k.numpy(), v.numpy(), m.numpy(), 0.25, do.numpy(), dtype=np.float64)
+    for got, want in ((dq, qr.grad), (dk, kr.grad), (dv, vr.grad)):
+        assert np.abs(got - want.numpy()).max() < 1e-11
+
+
+def test_elementwise_rows_without_keys_give_zero():
+    g = torch.Generator().manual_seed(6)
+    q, k, v = [torch.randn(1, 1, 64, 8, generator=g).numpy() for _ in range(3)]
+    m = np.ones((1, 1, 64, 64), dtype=bool)
+    m[0, 0, 5, :] = False
+    o, lse = orc.naive_attention(q, k, v, m, 0.5, return_lse=True)
+    assert np.all(o[0, 0, 5] == 0) and lse[0, 0, 5] == -np.inf and np.isfinite(lse[0, 0, 4])

@@ -95,3 +95,33 @@ def test_dense_reduce_and_expand_roundtrip():
     assert np.array_equal(orc.reduce_dense_mask(dense), block)
     d = np.zeros((1, 1, 128, 128), dtype=bool); d[0, 0, 70, 3] = True
     assert orc.reduce_dense_mask(d).tolist() == [[[[False, False], [True, False]]]]
+
+
+def test_pack_mask_tiles_format():
+    """Packed-tile format: one slot per kept tile in list order; word r bit c = element (r, c);
+    the transposed form lists tiles column block by column block with rows and columns swapped.
+    Checked by unpacking against the mask itself and against the kept-tile lists."""
+    rng = np.random.default_rng(3)
+    N, nb = 192, 3
+    dense = rng.random((1, 2, N, N)) < 0.4
+    dense[0, 0, :64, 64:128] = False                    # empty tile
+    dense[0, 0, 64:128, :64] = True                     # full tile
+    dense[0, 1, 128:, :] = False                        # empty row block
+    block = orc.reduce_dense_mask(dense)
+    for transpose in (False, True):
+        partial, words = orc.pack_mask_tiles(dense, transpose)
+        rp, ci = (orc.csc_from_block_mask(block) if transpose else orc.csr_from_block_mask(block))[:2]
+        assert len(partial) == len(ci) == words.shape[0]
+        t = 0
+        for bh in range(2):
+            for a in range(nb):
+                for j in range(rp[bh * nb + a], rp[bh * nb + a + 1]):
+                    c = ci[j]
+                    rb, cb = (c, a) if transpose else (a, c)
+                    tile = dense[0, bh, rb * 64:(rb + 1) * 64, cb * 64:(cb + 1) * 64]
+                    tile = tile.T if transpose else tile
+                    unpacked = (words[t][:, None] >> np.arange(64, dtype=np.uint64)[None, :]) & np.uint64(1)
+                    assert np.array_equal(unpacked.astype(bool), tile)
+                    assert partial[t] == (0 if tile.all() else 1)
+                    t += 1
+        assert t == len(partial)
