@@ -95,11 +95,12 @@ int bsattn_fwd_workspace(int B, int H, int N, int D, size_t* bytes) {
   return BSATTN_OK;
 }
 
-int bsattn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
-               const int32_t* row_ptr, const int32_t* col_idx, int Bm, int Hm, int B, int H, int N,
-               int D, int dtype, int out_dtype, float sm_scale, const int64_t* q_strides,
-               const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides,
-               void* workspace, size_t workspace_bytes, void* stream) {
+static int fwd_common(const void* q, const void* k, const void* v, void* o, float* lse,
+                      const int32_t* row_ptr, const int32_t* col_idx, const uint8_t* tile_partial,
+                      const uint64_t* tile_bits, int Bm, int Hm, int B, int H, int N,
+                      int D, int dtype, int out_dtype, float sm_scale, const int64_t* q_strides,
+                      const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides,
+                      void* workspace, size_t workspace_bytes, void* stream) {
   if (q == nullptr || k == nullptr || v == nullptr || o == nullptr || row_ptr == nullptr || col_idx == nullptr)
     return BSATTN_ERR_NULL;
   int rc = check_attn(Bm, Hm, B, H, N, D, dtype, out_dtype);
@@ -113,7 +114,29 @@ int bsattn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
   s.B = B; s.H = H; s.N = N; s.D = D; s.Bm = Bm; s.Hm = Hm; s.dtype = dtype; s.out_dtype = out_dtype;
   s.sm_scale = sm_scale;
   for (int i = 0; i < 3; ++i) { s.qs[i] = q_strides[i]; s.ks[i] = k_strides[i]; s.vs[i] = v_strides[i]; s.os[i] = o_strides[i]; s.dos[i] = 0; }
-  return launch_fwd(q, k, v, o, lse, row_ptr, col_idx, s, workspace, (hipStream_t)stream);
+  return launch_fwd(q, k, v, o, lse, row_ptr, col_idx, tile_partial, tile_bits, s, workspace, (hipStream_t)stream);
+}
+
+int bsattn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
+               const int32_t* row_ptr, const int32_t* col_idx, int Bm, int Hm, int B, int H, int N,
+               int D, int dtype, int out_dtype, float sm_scale, const int64_t* q_strides,
+               const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides,
+               void* workspace, size_t workspace_bytes, void* stream) {
+  return fwd_common(q, k, v, o, lse, row_ptr, col_idx, nullptr, nullptr, Bm, Hm, B, H, N, D, dtype, out_dtype,
+                    sm_scale, q_strides, k_strides, v_strides, o_strides, workspace, workspace_bytes, stream);
+}
+
+int bsattn_fwd_elementwise(const void* q, const void* k, const void* v, void* o, float* lse,
+                           const int32_t* row_ptr, const int32_t* col_idx, const uint8_t* tile_partial,
+                           const uint64_t* tile_bits, int Bm, int Hm, int B, int H, int N,
+                           int D, int dtype, int out_dtype, float sm_scale, const int64_t* q_strides,
+                           const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides,
+                           void* workspace, size_t workspace_bytes, void* stream) {
+  if (tile_partial == nullptr || tile_bits == nullptr) return BSATTN_ERR_NULL;
+  if (((uintptr_t)tile_bits & 7) != 0) return BSATTN_ERR_STRIDE;
+  return fwd_common(q, k, v, o, lse, row_ptr, col_idx, tile_partial, tile_bits, Bm, Hm, B, H, N, D, dtype,
+                    out_dtype, sm_scale, q_strides, k_strides, v_strides, o_strides, workspace, workspace_bytes,
+                    stream);
 }
 
 int bsattn_bwd_workspace(int B, int H, int N, int D, size_t* bytes) {

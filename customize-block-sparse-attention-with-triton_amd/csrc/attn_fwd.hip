@@ -34,6 +34,8 @@ namespace bsattn {
 struct FwdParams {
   const void* q; const void* k; const void* v; void* o; float* lse;
   const int32_t* row_ptr; const int32_t* col_idx;
+  const unsigned char* tile_partial;        // elementwise masks: per kept tile, 1 = only partly set
+  const unsigned long long* tile_bits;      // ... and its 64 row words (bit c = column c)
   float* ws;                       // partial slots of row blocks shared between workgroups
   unsigned long long* flags;       // one per slot: holds `epoch` once the slot's part is complete
   unsigned long long epoch;        // distinguishes this launch's flags from stale contents
@@ -75,7 +77,9 @@ __device__ __forceinline__ void* out_base(const FwdParams& prm, int b, int h) {
 
 // Rare path of the softmax: re-centre the reference exponent of one query block on the row
 // maximum of the current tile and redo the tile's numerators.
-template <int DB, bool FOLD>
+// With elementwise masks (EW) a query may have had nothing but masked keys so far (l == 0, or the
+// whole tile masked: maximum -inf): such a lane takes the tile's maximum as its first reference.
+template <int DB, bool FOLD, bool EW>
 __device__ __forceinline__ void recentre(floatx16& s0, floatx16& s1, floatx16 (&oacc)[DB][2], int qb, float qk_scale,
                                       float& m, float& l, uintx4& mfrag, bool fresh, int g) {
   float mx = max3f(s0[0], s0[1], s0[2]);
@@ -87,10 +91,16 @@ __device__ __forceinline__ void recentre(floatx16& s0, floatx16& s1, floatx16 (&
   mx = xhalf_max(fmaxf(mx, s1[15]));
   // exponent of the largest entry relative to the current reference
   const float smax = FOLD ? mx : __builtin_fmaf(mx, qk_scale, -m);
-  const float delta = fresh ? smax : fmaxf(smax, 0.f);
+  float delta = fresh ? smax : fmaxf(smax, 0.f);
+  bool nomass = false;
+  if constexpr (EW) {
+    nomass = !fresh && l == 0.f;
+    if (nomass) delta = smax;
+    if (smax == -INFINITY) delta = 0.f;
+  }
   m += delta;
   if (!fresh) {
-    const float alpha = __builtin_amdgcn_exp2f(-delta);
+    const float alpha = nomass ? 1.0f : __builtin_amdgcn_exp2f(-delta);
     l *= alpha;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
@@ -127,14 +137,15 @@ template <int D> struct FwdCfg {
   static constexpr int WAVE_LDS = 2 * TILE_BYTES;           // K buffer + V buffer
   static constexpr int ML_BYTES = NW * 2 * 64 * 4 + 64;     // exchange of (m, l) per query + the tile counter
   static constexpr int COLS_CAP = 2048;                     // column indices of the range kept in LDS
-  static constexpr int LDS_BYTES = NW * WAVE_LDS + ML_BYTES + COLS_CAP * 4;
+  static constexpr int BITS_OFF = NW * WAVE_LDS + ML_BYTES + COLS_CAP * 4;   // mask words of the current tile, 512 bytes per wavefront
+  static constexpr int LDS_BYTES = BITS_OFF + NW * 512;
   static constexpr int R = TILE_BYTES / 256;                // accumulator registers exchanged per round
   static constexpr int ROUNDS = D / R;
   static constexpr int QPW = (R / 4) / NW;                  // output quads per wavefront and round
   static constexpr int SHORT_ROW = 6 * NW;                  // row blocks up to this many tiles may go to one wavefront
 };
 
-template <int D, bool BF16, bool ROWS>
+template <int D, bool BF16, bool ROWS, bool EW>
 __global__ __launch_bounds__(FwdCfg<D>::NW * 64, FwdCfg<D>::WG_PER_CU)
 void fwd_kernel(const FwdParams prm) {
   using C = FwdCfg<D>;
@@ -211,9 +222,20 @@ void fwd_kernel(const FwdParams prm) {
   auto v_copy = [&](const unsigned short* tile, int j) {
     tile_load_async_one(tile + (int64_t)j * RPI * prm.vs[2], voff[0], lds_v_addr + j * 1024);
   };
-  auto k_copy_all = [&](const unsigned short* tile) {
+  const unsigned lds_bits_addr = (unsigned)(uintptr_t)(lds_ptr_t)lds + C::BITS_OFF + w * 512;
+  const unsigned long long* lds_bits = reinterpret_cast<const unsigned long long*>(lds + C::BITS_OFF + w * 512);
+  constexpr int KOPS = CPR + (EW ? 2 : 0);      // instructions of one K copy
+  // copy of the K tile `tile` = entry t of the kept-tile list (EW: with its 512 bytes of mask words)
+  auto k_copy_all = [&](const unsigned short* tile, int t) {
 #pragma unroll
     for (int j = 0; j < CPR; ++j) k_copy(tile, j);
+    if constexpr (EW) {
+      const unsigned long long* src = prm.tile_bits + (int64_t)t * 64;
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2"
+                     :: "s"(lds_bits_addr + j * 256), "v"(4u * (unsigned)lane + 256u * j), "s"(src) : "memory", "m0");
+    }
   };
   auto v_copy_all = [&](const unsigned short* tile) {
 #pragma unroll
@@ -294,7 +316,7 @@ void fwd_kernel(const FwdParams prm) {
   // numerators of block 1, [4] second product of block 1.  Operand fragments are read from LDS
   // once, all at once (the read latency is a multiple of an MFMA's issue interval), and serve
   // both query blocks.
-  auto tile = [&](bool has1, int cbn, bool copy_v, auto&& mid) {
+  auto tile = [&](bool has1, int cbn, int tn, bool copy_v, bool partial, auto&& mid) {
     uintx4 kfr[2][KS], vfr[4][DB];
     uintx4 pf[4][2];  // P^T operand fragments: [16-key slice][qb]
     auto scores = [&](int qb, floatx16& s0, floatx16& s1) {   // S^T[.][qb] = K Q[qb]^T (- m_i when FOLD)
@@ -344,8 +366,8 @@ void fwd_kernel(const FwdParams prm) {
     // finite), some P left the safe fp16 range: recentre() moves m_i to the tile's row maximum
     // and the numerators are redone from the scores, which are still live.
     auto settle = [&](int qb, floatx16& s0, floatx16& s1, float lnew) {
-      if (__any(fresh || !(lnew - l_i[qb] < 16384.0f))) {
-        recentre<DB, FOLD>(s0, s1, oacc, qb, qk_scale, m_i[qb], l_i[qb], mfrag[qb], fresh, g);
+      if (__any(fresh || (EW && l_i[qb] == 0.f) || !(lnew - l_i[qb] < 16384.0f))) {
+        recentre<DB, FOLD, EW>(s0, s1, oacc, qb, qk_scale, m_i[qb], l_i[qb], mfrag[qb], fresh, g);
         lnew = softmax_tile<FOLD>(s0, s1, qk_scale, m_i[qb], l_i[qb], pf, qb);
       }
       l_i[qb] = lnew;
@@ -357,14 +379,31 @@ void fwd_kernel(const FwdParams prm) {
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
       for (int s = 0; s < KS; ++s) kfr[kb][s] = *reinterpret_cast<const uintx4*>(lds_k + kaddr[kb][s]);
+    // EW: the 64 mask bits of this lane's two queries, shifted so that bit 8(i/4) + i%4 (+ 32 for
+    // the second key block) is the key of score register i
+    unsigned long long mw0 = 0ull, mw1 = 0ull;
+    if constexpr (EW) {
+      if (partial) { mw0 = lds_bits[ln] >> (4 * g); mw1 = lds_bits[32 + ln] >> (4 * g); }
+    }
     lds_wait();      // the K fragments have arrived: the K buffer is free
     mid();
-    if (has1) k_copy_all(kg + (int64_t)cbn * 64 * prm.ks[2]);
+    if (has1) k_copy_all(kg + (int64_t)cbn * 64 * prm.ks[2], tn);
+    auto mask_scores = [&](floatx16& s0, floatx16& s1, unsigned long long mw) {
+      const unsigned lo = (unsigned)mw, hi = (unsigned)(mw >> 32);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const unsigned bit = 1u << (8 * (i / 4) + (i % 4));
+        s0[i] = (lo & bit) ? s0[i] : -INFINITY;
+        s1[i] = (hi & bit) ? s1[i] : -INFINITY;
+      }
+    };
     // [1]
     scores(0, sa0, sa1);
+    if constexpr (EW) { if (partial) mask_scores(sa0, sa1, mw0); }
     __builtin_amdgcn_sched_barrier(0);
     // [2]
     scores(1, sb0, sb1);
+    if constexpr (EW) { if (partial) mask_scores(sb0, sb1, mw1); }
     float lnew0 = softmax_tile<FOLD>(sa0, sa1, qk_scale, m_i[0], l_i[0], pf, 0);
 #pragma unroll
     for (int it = 0; it < 2 * KS + (FOLD ? 2 : 0); ++it) {
@@ -373,7 +412,7 @@ void fwd_kernel(const FwdParams prm) {
     }
     __builtin_amdgcn_sched_barrier(0);
     settle(0, sa0, sa1, lnew0);
-    if (has1) wait_vm<CPR>(); else wait_vm<0>();  // V(cur) has landed (K(nxt) may be in flight)
+    if (has1) wait_vm<KOPS>(); else wait_vm<0>();  // V(cur) has landed (K(nxt) may be in flight)
     read_v();
     lds_wait();      // the V fragments have arrived: the V buffer is free
     if (copy_v) v_copy_all(vg + (int64_t)cbn * 64 * prm.vs[2]);
@@ -398,8 +437,20 @@ void fwd_kernel(const FwdParams prm) {
   // The column indices of the range are staged in LDS: a scalar load per tile would put its whole
   // latency in front of the tile's first LDS wait (scalar loads return out of order, so any wait
   // on the shared counter becomes a wait for all of them).
+  typedef const unsigned char __attribute__((address_space(4)))* cbyte_ptr_t;
+  // entry t of the column list as staged: column block in the low bits, "partly set" in bit 30
+  auto flagged_col = [&](int t) {
+    int c = cols[t];
+    if constexpr (EW) c |= (int)((cbyte_ptr_t)(uintptr_t)prm.tile_partial)[t] << 30;
+    return c;
+  };
+  constexpr int COL_MASK = 0x3fffffff;
   auto stage_cols = [&](int t_lo, int t_hi) {
-    for (int i = threadIdx.x; i < t_hi - t_lo && i < C::COLS_CAP; i += NW * 64) lcols[i] = prm.col_idx[t_lo + i];
+    for (int i = threadIdx.x; i < t_hi - t_lo && i < C::COLS_CAP; i += NW * 64) {
+      int c = prm.col_idx[t_lo + i];
+      if constexpr (EW) c |= (int)prm.tile_partial[t_lo + i] << 30;     // EW: "partly set" rides in bit 30
+      lcols[i] = c;
+    }
   };
 
   // Whole row blocks [r_lo, r_hi), one wavefront each: handed out through the LDS counter *rctr
@@ -419,18 +470,19 @@ void fwd_kernel(const FwdParams prm) {
       const int tn = tick_next < r_hi ? rp[row_next] : 0;
       const bool next_has = tick_next < r_hi && rp[row_next + 1] > tn;
       if (ta < tb) {
+        int cx = __builtin_amdgcn_readfirstlane(col_of(ta));      // current tile: column block | flag
         if (kdone != ta) {
-          const int cb = __builtin_amdgcn_readfirstlane(col_of(ta));
-          k_copy_all(kg + (int64_t)cb * 64 * prm.ks[2]);
-          v_copy_all(vg + (int64_t)cb * 64 * prm.vs[2]);
+          k_copy_all(kg + (int64_t)(cx & COL_MASK) * 64 * prm.ks[2], ta);
+          v_copy_all(vg + (int64_t)(cx & COL_MASK) * 64 * prm.vs[2]);
         }
         reset_acc();
         load_q(row);
         for (int j = ta; j < tb; ++j) {
           const bool last = j + 1 == tb;
           const bool has1 = !last || next_has;
-          const int cbn = has1 ? __builtin_amdgcn_readfirstlane(col_of(last ? tn : j + 1)) : 0;
-          tile(has1, cbn, has1, [] {});
+          const int cxn = has1 ? __builtin_amdgcn_readfirstlane(col_of(last ? tn : j + 1)) : 0;
+          tile(has1, cxn & COL_MASK, last ? tn : j + 1, has1, (cx >> 30) != 0, [] {});
+          cx = cxn;
         }
         kdone = next_has ? tn : -1;
         // normalise and write the row block
@@ -439,7 +491,7 @@ void fwd_kernel(const FwdParams prm) {
         for (int qb = 0; qb < 2; ++qb) lsum[qb] = l_i[qb] + __shfl_xor(l_i[qb], 32);
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
-          const float inv = 1.0f / lsum[qb];
+          const float inv = lsum[qb] > 0.f ? 1.0f / lsum[qb] : 0.f;      // no unmasked key at all: O = 0
           const int64_t qrow = (int64_t)(row * 64 + qb * 32 + ln);
 #pragma unroll
           for (int db = 0; db < DB; ++db)
@@ -449,7 +501,8 @@ void fwd_kernel(const FwdParams prm) {
                                oacc[db][qb][4 * i4] * inv, oacc[db][qb][4 * i4 + 1] * inv,
                                oacc[db][qb][4 * i4 + 2] * inv, oacc[db][qb][4 * i4 + 3] * inv);
           if (prm.lse != nullptr && g == 0)
-            prm.lse[((int64_t)bh * prm.N) + qrow] = (m_i[qb] + __builtin_amdgcn_logf(lsum[qb])) * 0.6931471805599453f;
+            prm.lse[((int64_t)bh * prm.N) + qrow] =
+                lsum[qb] > 0.f ? (m_i[qb] + __builtin_amdgcn_logf(lsum[qb])) * 0.6931471805599453f : -INFINITY;
         }
       } else {
         // row block without kept tiles: O = 0, lse = -inf
@@ -489,7 +542,7 @@ void fwd_kernel(const FwdParams prm) {
     stage_cols(t_lo, rp[r_hi]);
     if (threadIdx.x == 0) *ctr = r_lo + 2 * NW;
     __syncthreads();
-    auto col_of = [&](int t) { return t - t_lo < C::COLS_CAP ? lcols[t - t_lo] : (int)cols[t]; };
+    auto col_of = [&](int t) { return t - t_lo < C::COLS_CAP ? lcols[t - t_lo] : flagged_col(t); };
     run_rows(r_lo, r_hi, ctr, col_of);
   } else {
     // ================= all wavefronts on one row block at a time =================
@@ -510,7 +563,7 @@ void fwd_kernel(const FwdParams prm) {
     stage_cols(g0, g1);
     if (threadIdx.x == 0) { ctr[0] = g0 + 2 * NW; ctr[3] = 0; }
     __syncthreads();
-    auto col_of = [&](int t) { return t - g0 < C::COLS_CAP ? lcols[t - g0] : (int)cols[t]; };
+    auto col_of = [&](int t) { return t - g0 < C::COLS_CAP ? lcols[t - g0] : flagged_col(t); };
     int cur = g0 + w, nxt = g0 + NW + w;      // the first two rounds are fixed
     int cb_nxt = nxt < g1 ? __builtin_amdgcn_readfirstlane(col_of(nxt)) : 0;   // column block of tile nxt
     int kdone = -1, vdone = -1;
@@ -555,9 +608,9 @@ void fwd_kernel(const FwdParams prm) {
       const bool mine = cur < seg_b;      // this wavefront processes at least one tile of the row block
       reset_acc();
       if (mine) {
-        const int cbc = __builtin_amdgcn_readfirstlane(col_of(cur));
-        if (kdone != cur) { k_copy_all(kg + (int64_t)cbc * 64 * prm.ks[2]); kdone = cur; }
-        if (vdone != cur) { v_copy_all(vg + (int64_t)cbc * 64 * prm.vs[2]); vdone = cur; }
+        int cx = __builtin_amdgcn_readfirstlane(col_of(cur));     // current tile: column block | flag
+        if (kdone != cur) { k_copy_all(kg + (int64_t)(cx & COL_MASK) * 64 * prm.ks[2], cur); kdone = cur; }
+        if (vdone != cur) { v_copy_all(vg + (int64_t)(cx & COL_MASK) * 64 * prm.vs[2]); vdone = cur; }
         load_q(r);
         while (cur < seg_b) {
           // draw the tile after next; the value is picked up inside the tile
@@ -565,13 +618,14 @@ void fwd_kernel(const FwdParams prm) {
           if (lane == 0) drawn = atomicAdd(ctr, 1);
           const bool has1 = nxt < g1, copy_v = nxt < seg_b;
           int nn = 0, cb_nn_v = 0;
-          tile(has1, cb_nxt, copy_v, [&] {
+          tile(has1, cb_nxt & COL_MASK, nxt, copy_v, (cx >> 30) != 0, [&] {
             nn = __builtin_amdgcn_readfirstlane(drawn);
             cb_nn_v = nn < g1 ? col_of(nn) : 0;     // looked up now, needed at the end of the tile
           });
           if (has1) kdone = nxt;
           if (copy_v) vdone = nxt;
           cur = nxt;
+          cx = cb_nxt;
           nxt = nn;
           cb_nxt = __builtin_amdgcn_readfirstlane(cb_nn_v);
         }  // tiles of this wavefront
@@ -588,8 +642,9 @@ void fwd_kernel(const FwdParams prm) {
         if (g == 0) {
 #pragma unroll
           for (int qb = 0; qb < 2; ++qb) {
-            ml[(w * 2 + 0) * 64 + qb * 32 + ln] = mine ? m_i[qb] : -INFINITY;
-            ml[(w * 2 + 1) * 64 + qb * 32 + ln] = mine ? lsum[qb] : 0.f;
+            const bool mass = mine && lsum[qb] > 0.f;
+            ml[(w * 2 + 0) * 64 + qb * 32 + ln] = mass ? m_i[qb] : -INFINITY;
+            ml[(w * 2 + 1) * 64 + qb * 32 + ln] = mass ? lsum[qb] : 0.f;
           }
         }
         // A row block cut by range boundaries is finished by the workgroup that holds its first
@@ -650,7 +705,7 @@ void fwd_kernel(const FwdParams prm) {
               for (int e = 0; e < 4; ++e) x[e] += wgt[pw][qb] * src[(4 * quad + e) * 64 + lane];
             }
             if (full) {
-              const float inv = 1.0f / L[qb];
+              const float inv = L[qb] > 0.f ? 1.0f / L[qb] : 0.f;
               const int64_t qrow = (int64_t)(r * 64 + qb * 32 + ln);
               store_out4<BF16>(obase, qrow * prm.os[2] + 32 * db + 8 * i4 + 4 * g, prm.out_f32, x[0] * inv, x[1] * inv,
                                x[2] * inv, x[3] * inv);
@@ -668,7 +723,7 @@ void fwd_kernel(const FwdParams prm) {
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb)
               prm.lse[((int64_t)bh * prm.N) + (int64_t)(r * 64 + qb * 32 + ln)] =
-                  (M[qb] + __builtin_amdgcn_logf(L[qb])) * 0.6931471805599453f;
+                  L[qb] > 0.f ? (M[qb] + __builtin_amdgcn_logf(L[qb])) * 0.6931471805599453f : -INFINITY;
           }
         } else if (publish) {
           if (w == 0 && g == 0) {
@@ -716,9 +771,9 @@ void fwd_kernel(const FwdParams prm) {
             float sc_own[2], sc_p[2];
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb) {
-              const float mn = fmaxf(M[qb], mp[qb]);
-              sc_own[qb] = __builtin_amdgcn_exp2f(M[qb] - mn);
-              sc_p[qb] = __builtin_amdgcn_exp2f(mp[qb] - mn);
+              const float mn = fmaxf(M[qb], mp[qb]);     // a side without mass has maximum -inf and weight 0
+              sc_own[qb] = M[qb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(M[qb] - mn);
+              sc_p[qb] = mp[qb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mp[qb] - mn);
               L[qb] = L[qb] * sc_own[qb] + lp[qb] * sc_p[qb];
               M[qb] = mn;
             }
@@ -738,7 +793,7 @@ void fwd_kernel(const FwdParams prm) {
             for (int tq = 0; tq < C::QPW; ++tq) {
               const int idx0 = rd * C::R + 4 * (w * C::QPW + tq);
               const int db = idx0 / 32, qb = (idx0 / 16) & 1, i4 = (idx0 & 15) / 4;
-              const float inv = 1.0f / L[qb];
+              const float inv = L[qb] > 0.f ? 1.0f / L[qb] : 0.f;
               const int64_t qrow = (int64_t)(r * 64 + qb * 32 + ln);
               store_out4<BF16>(obase, qrow * prm.os[2] + 32 * db + 8 * i4 + 4 * g, prm.out_f32,
                                keep[rd][tq][0] * inv + bad, keep[rd][tq][1] * inv + bad, keep[rd][tq][2] * inv + bad,
@@ -748,7 +803,7 @@ void fwd_kernel(const FwdParams prm) {
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb)
               prm.lse[((int64_t)bh * prm.N) + (int64_t)(r * 64 + qb * 32 + ln)] =
-                  (M[qb] + __builtin_amdgcn_logf(L[qb])) * 0.6931471805599453f + bad;
+                  (L[qb] > 0.f ? (M[qb] + __builtin_amdgcn_logf(L[qb])) * 0.6931471805599453f : -INFINITY) + bad;
           }
           // every wavefront has read the flags: put them back to zero, so that a replay of this
           // launch (same epoch) does not take this launch's parts for its own
@@ -809,30 +864,31 @@ size_t fwd_workspace_bytes(int B, int H, int N, int D) {
 // wavefront takes whole row blocks, which needs no merge and no second kernel.
 static bool rows_mode(const FwdParams& prm) { return prm.nb >= 8 * prm.W; }
 
-template <int D, bool BF16>
+template <int D, bool BF16, bool EW>
 static void launch_fwd_t(const FwdParams& prm, int BH, hipStream_t st) {
   using C = FwdCfg<D>;
   static bool configured = false;   // raising the dynamic LDS limit is idempotent
   if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<D, BF16, false>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<D, BF16, false, EW>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<D, BF16, true>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<D, BF16, true, EW>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
     configured = true;
   }
   if (rows_mode(prm)) {
-    hipLaunchKernelGGL((fwd_kernel<D, BF16, true>), dim3(prm.W * BH), dim3(C::NW * 64), C::LDS_BYTES, st, prm);
+    hipLaunchKernelGGL((fwd_kernel<D, BF16, true, EW>), dim3(prm.W * BH), dim3(C::NW * 64), C::LDS_BYTES, st, prm);
   } else {
-    hipLaunchKernelGGL((fwd_kernel<D, BF16, false>), dim3(prm.W * BH), dim3(C::NW * 64), C::LDS_BYTES, st, prm);
+    hipLaunchKernelGGL((fwd_kernel<D, BF16, false, EW>), dim3(prm.W * BH), dim3(C::NW * 64), C::LDS_BYTES, st, prm);
   }
 }
 
 int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
-               const int32_t* row_ptr, const int32_t* col_idx, const AttnShape& s, void* ws,
-               hipStream_t st) {
+               const int32_t* row_ptr, const int32_t* col_idx, const uint8_t* tile_partial,
+               const uint64_t* tile_bits, const AttnShape& s, void* ws, hipStream_t st) {
   FwdParams prm;
   prm.q = q; prm.k = k; prm.v = v; prm.o = o; prm.lse = lse;
   prm.row_ptr = row_ptr; prm.col_idx = col_idx; prm.ws = (float*)ws;
+  prm.tile_partial = tile_partial; prm.tile_bits = (const unsigned long long*)tile_bits;
   prm.B = s.B; prm.H = s.H; prm.N = s.N; prm.nb = s.N / 64; prm.Bm = s.Bm; prm.Hm = s.Hm;
   prm.W = groups_per_head(s.B, s.H, prm.nb, s.D);
   // with two workgroups per compute unit the first-comers are faster: tell the kernel which they are
@@ -843,10 +899,18 @@ int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
   prm.qk_scale = s.sm_scale * 1.4426950408889634f;
   for (int i = 0; i < 3; ++i) { prm.qs[i] = s.qs[i]; prm.ks[i] = s.ks[i]; prm.vs[i] = s.vs[i]; prm.os[i] = s.os[i]; }
   const bool bf = s.dtype == BSATTN_BF16;
-  if (s.D == 64 && !bf) launch_fwd_t<64, false>(prm, s.B * s.H, st);
-  else if (s.D == 64 && bf) launch_fwd_t<64, true>(prm, s.B * s.H, st);
-  else if (s.D == 128 && !bf) launch_fwd_t<128, false>(prm, s.B * s.H, st);
-  else launch_fwd_t<128, true>(prm, s.B * s.H, st);
+  const int BH = s.B * s.H;
+  if (tile_bits == nullptr) {
+    if (s.D == 64 && !bf) launch_fwd_t<64, false, false>(prm, BH, st);
+    else if (s.D == 64 && bf) launch_fwd_t<64, true, false>(prm, BH, st);
+    else if (s.D == 128 && !bf) launch_fwd_t<128, false, false>(prm, BH, st);
+    else launch_fwd_t<128, true, false>(prm, BH, st);
+  } else {   // elementwise mask: kernels that apply the packed mask words inside partly set tiles
+    if (s.D == 64 && !bf) launch_fwd_t<64, false, true>(prm, BH, st);
+    else if (s.D == 64 && bf) launch_fwd_t<64, true, true>(prm, BH, st);
+    else if (s.D == 128 && !bf) launch_fwd_t<128, false, true>(prm, BH, st);
+    else launch_fwd_t<128, true, true>(prm, BH, st);
+  }
   return launch_status();
 }
 

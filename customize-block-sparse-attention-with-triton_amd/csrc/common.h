@@ -29,8 +29,8 @@ struct AttnShape {
 // attn_fwd.hip
 size_t fwd_workspace_bytes(int B, int H, int N, int D);
 int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
-               const int32_t* row_ptr, const int32_t* col_idx, const AttnShape& s, void* ws,
-               hipStream_t st);
+               const int32_t* row_ptr, const int32_t* col_idx, const uint8_t* tile_partial,
+               const uint64_t* tile_bits, const AttnShape& s, void* ws, hipStream_t st);
 
 // attn_bwd.hip
 size_t bwd_workspace_bytes(int B, int H, int N, int D);

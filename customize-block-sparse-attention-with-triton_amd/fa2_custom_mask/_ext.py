@@ -27,6 +27,8 @@ _SIGNATURES = {
     "bsattn_fwd_workspace": ([_i, _i, _i, _i, ctypes.POINTER(ctypes.c_size_t)], _i),
     "bsattn_fwd": ([_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f,
                     _p, _p, _p, _p, _p, ctypes.c_size_t, _p], _i),
+    "bsattn_fwd_elementwise": ([_p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f,
+                                _p, _p, _p, _p, _p, ctypes.c_size_t, _p], _i),
     "bsattn_bwd_workspace": ([_i, _i, _i, _i, ctypes.POINTER(ctypes.c_size_t)], _i),
     "bsattn_bwd": ([_p] * 13 + [_i] * 8 + [_f] + [_p] * 5 + [_p, ctypes.c_size_t, _p], _i),
     "bsattn_reorder": ([_p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p], _i),

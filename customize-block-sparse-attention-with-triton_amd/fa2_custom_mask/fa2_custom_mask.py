@@ -72,12 +72,15 @@ def _forward(q, k, v, lists, sm_scale, out_dtype, want_lse):
     lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device) if want_lse else None  # :70
     wsb = _ext.fwd_workspace(B, H, N, D)
     ws = torch.empty(wsb, dtype=torch.uint8, device=q.device)
-    rc = _ext.lib().bsattn_fwd(
-        q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr() if want_lse else None,
-        lists.row_ptr.data_ptr(), lists.col_idx.data_ptr(), lists.Bm, lists.Hm, B, H, N, D,
-        _ext.dtype_code(q.dtype), _ext.dtype_code(out_dtype), float(sm_scale),
-        _ext.strides4(q), _ext.strides4(k), _ext.strides4(v), _ext.strides4(o),
-        ws.data_ptr(), wsb, _ext.current_stream(q.device))
+    common = (lists.Bm, lists.Hm, B, H, N, D, _ext.dtype_code(q.dtype), _ext.dtype_code(out_dtype), float(sm_scale),
+              _ext.strides4(q), _ext.strides4(k), _ext.strides4(v), _ext.strides4(o),
+              ws.data_ptr(), wsb, _ext.current_stream(q.device))
+    ptrs = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr() if want_lse else None,
+            lists.row_ptr.data_ptr(), lists.col_idx.data_ptr())
+    if lists.bits is None:
+        rc = _ext.lib().bsattn_fwd(*ptrs, *common)
+    else:                                      # elementwise mask: exact inside partly set tiles
+        rc = _ext.lib().bsattn_fwd_elementwise(*ptrs, lists.partial.data_ptr(), lists.bits.data_ptr(), *common)
     _ext.check(rc, "bsattn_fwd")
     return o, lse
 

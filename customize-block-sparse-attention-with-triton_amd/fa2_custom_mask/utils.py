@@ -29,11 +29,13 @@ class TileLists:
     entries valid), counts int32 [2] = (G, T), groups int32 [Bm*Hm*nb, 5] (first G rows
     valid) or None."""
 
-    __slots__ = ("row_ptr", "col_idx", "groups", "counts", "Bm", "Hm", "nb")
+    __slots__ = ("row_ptr", "col_idx", "groups", "counts", "Bm", "Hm", "nb", "partial", "bits")
 
     def __init__(self, row_ptr, col_idx, groups, counts, Bm, Hm, nb):
         self.row_ptr, self.col_idx, self.groups, self.counts = row_ptr, col_idx, groups, counts
         self.Bm, self.Hm, self.nb = Bm, Hm, nb
+        # elementwise masks only: per kept tile "partly set" flag and packed 64 x 64 bits
+        self.partial, self.bits = None, None
 
 
 def _check_mask(mask):
@@ -160,5 +162,7 @@ def mask_to_lists(mask, N, transpose=False):
     lists = lists_cache.get(mask, N, transpose)
     if lists is None:
         lists = block_mask_to_lists(to_block_mask(mask, N), transpose=transpose)
+        if mask.shape[2] == N and N != N // TILE:          # elementwise form: exact inside tiles
+            lists.partial, lists.bits = pack_mask_tiles(mask, lists, transpose=transpose)
         lists_cache.put(mask, N, transpose, lists)
     return lists

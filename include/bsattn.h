@@ -125,6 +125,21 @@ int bsattn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                void* stream);
 
 /* ------------------------------------------------------------------------------------
+ * Forward with an elementwise mask: as bsattn_fwd, and inside the kept tiles flagged in
+ * tile_partial the scores of unset elements are -inf (kernel-test.py:38; the semantics
+ * the reference's unused inner loop fa2_fwd.py:67-73 intends).  tile_partial / tile_bits
+ * as made by bsattn_pack_mask_tiles for the same lists.  Query rows without any set
+ * element give O = 0, lse = -inf.
+ * ---------------------------------------------------------------------------------- */
+int bsattn_fwd_elementwise(const void* q, const void* k, const void* v, void* o, float* lse,
+                           const int32_t* row_ptr, const int32_t* col_idx,
+                           const uint8_t* tile_partial, const uint64_t* tile_bits, int Bm, int Hm,
+                           int B, int H, int N, int D, int dtype, int out_dtype, float sm_scale,
+                           const int64_t* q_strides, const int64_t* k_strides,
+                           const int64_t* v_strides, const int64_t* o_strides, void* workspace,
+                           size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------
  * Backward.  Replaces _attn_bwd_preprocess and _attn_bwd (fa2_custom_mask/fa2_bwd.py:5-19,
  * 140-285) as launched from _attention.backward (fa2_custom_mask/fa2_custom_mask.py:97-155).
  * The gradient algebra is the reference's (fa2_bwd.py:17,57-74,117-130,232,284) evaluated

@@ -1,0 +1,90 @@
+"""GPU parity of the elementwise-mask path (exact semantics inside partly set tiles) against the
+CPU oracle's naive masked softmax (kernel-test.py:37-40 with the mask used as it is)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import bsattn_oracle as orc
+from helpers import make_qkv, errors, f32
+
+pytestmark = pytest.mark.gpu
+
+MAXABS = {torch.float16: 2e-2, torch.bfloat16: 3e-2}
+
+
+def token_causal(N):
+    return torch.tril(torch.ones(N, N, dtype=torch.bool)).reshape(1, 1, N, N)
+
+
+def check_forward(dev, B, H, N, D, dtype, mask, seed, q_gain=1.0):
+    import fa2_custom_mask as fm
+    q, k, v = make_qkv(B, H, N, D, dtype, seed)
+    q = (q.float() * q_gain).to(dtype)
+    sc = 1.0 / np.sqrt(D)
+    o_ref, lse_ref = orc.naive_attention(f32(q), f32(k), f32(v), mask.numpy(), sc, return_lse=True)
+    o, lse = fm.flash_attention_custom_mask_lse(q.to(dev), k.to(dev), v.to(dev), mask.to(dev), sc, out_fp32=True)
+    torch.cuda.synchronize()
+    ma, rl = errors(o, o_ref)
+    print("B%d H%d N%d D%d %s gain %.0f: max-abs %.3e rel-L2 %.3e" % (B, H, N, D, dtype, q_gain, ma, rl))
+    assert ma <= MAXABS[dtype] and rl <= 1e-3
+    fin = np.isfinite(lse_ref)
+    l = lse.cpu().numpy()
+    assert np.array_equal(np.isfinite(l), fin)
+    assert np.abs(l[fin] - lse_ref[fin]).max() <= 2e-3 * max(1.0, q_gain)
+    assert float(np.abs(f32(o)[~fin]).max() if (~fin).any() else 0.0) == 0.0
+    return o
+
+
+@pytest.mark.parametrize("D,dtype", [(64, torch.float16), (128, torch.bfloat16), (64, torch.bfloat16), (128, torch.float16)])
+def test_token_causal_mask(dev, D, dtype):
+    """Token-level causal mask: every diagonal tile is partly set, tiles below are full."""
+    check_forward(dev, 1, 2, 512, D, dtype, token_causal(512), 51)
+
+
+@pytest.mark.parametrize("D,dtype", [(64, torch.float16), (128, torch.bfloat16)])
+def test_random_elementwise_masks(dev, D, dtype):
+    g = torch.Generator().manual_seed(52)
+    N = 512
+    m = torch.rand(2, 3, N, N, generator=g) < 0.5
+    m[0, 0, :, 64:128] = False                 # empty tiles
+    m[0, 1, 128:256, :] = True                 # full tiles
+    m[1, 2, 200:210, :] = False                # queries without any key
+    m[1, 0, :64, :] = False                    # a whole row block without keys
+    m[1, 1, 5, :] = False
+    m[1, 1, 5, 300] = True                     # one key only
+    check_forward(dev, 2, 3, N, D, dtype, m, 53)
+    check_forward(dev, 2, 3, N, D, dtype, m[:1, :1], 54)          # shared by all heads
+
+
+def test_first_tiles_masked_and_large_scores(dev):
+    """Queries whose first kept tiles are masked for them start without a reference exponent; with
+    large negative or positive scores afterwards nothing may underflow or overflow."""
+    g = torch.Generator().manual_seed(55)
+    N = 1024
+    m = torch.zeros(1, 1, N, N, dtype=torch.bool)
+    m[0, 0] = torch.rand(N, N, generator=g) < 0.3
+    m[0, 0, ::2, :448] = False                 # even queries: nothing in the first seven tiles
+    m[0, 0, 0, :] = False
+    m[0, 0, 0, N - 1] = True
+    for gain in (1.0, 8.0):
+        check_forward(dev, 1, 1, N, 64, torch.float16, m, 56, q_gain=gain)
+
+
+def test_many_heads_elementwise(dev):
+    """Row-block-per-wavefront mode (many heads) with partly set tiles."""
+    g = torch.Generator().manual_seed(57)
+    N = 512
+    m = (torch.rand(1, 1, N, N, generator=g) < 0.6) & token_causal(N)
+    m[0, 0, 70, :] = False
+    check_forward(dev, 4, 64, N, 64, torch.float16, m, 58)
+
+
+def test_tile_constant_elementwise_equals_block(dev):
+    import fa2_custom_mask as fm
+    from helpers import uniform_block_mask, same_up_to_rounding
+    N = 1024
+    block = uniform_block_mask(1, 2, N // 64, 0.4, 59)
+    dense = block.repeat_interleave(64, 2).repeat_interleave(64, 3)
+    q, k, v = [x.to(dev) for x in make_qkv(1, 2, N, 64, torch.float16, 60)]
+    assert same_up_to_rounding(fm.flash_attention_custom_mask(q, k, v, dense.to(dev), 0.125),
+                               fm.flash_attention_custom_mask(q, k, v, block.to(dev), 0.125))
