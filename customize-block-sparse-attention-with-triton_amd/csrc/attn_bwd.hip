@@ -25,6 +25,8 @@ struct BwdParams {
   const float* lse; float* delta;
   void* dq; void* dk; void* dv;
   const int32_t* row_ptr; const int32_t* col_idx; const int32_t* col_ptr; const int32_t* row_idx;
+  // elementwise masks: 64 words per entry of the row lists (bit = key) / of the column lists (bit = query)
+  const unsigned long long* bits_rows; const unsigned long long* bits_cols;
   int B, H, N, nb, Bm, Hm;
   int out_f32;
   float sm_scale, qk_scale;   // qk_scale = sm_scale * log2(e)
@@ -69,10 +71,11 @@ __global__ __launch_bounds__(256) void delta_kernel(const BwdParams prm) {
 // ---------------------------------------------------------------------------------------
 // helpers of the two walking kernels
 // ---------------------------------------------------------------------------------------
-template <int D> struct BwdCfg {
+template <int D, bool EW> struct BwdCfg {
   static constexpr int TILE_BYTES = 64 * 2 * D;
   static constexpr int STAT_BYTES = 2 * 64 * 4;                    // lse2[64] + delta[64] of a row block
-  static constexpr int STAGE_BYTES = 2 * TILE_BYTES + STAT_BYTES;  // two tiles (+ row statistics)
+  static constexpr int BITS_BYTES = EW ? 64 * 8 : 0;               // mask words of the tile (elementwise masks)
+  static constexpr int STAGE_BYTES = 2 * TILE_BYTES + STAT_BYTES + BITS_BYTES;  // two tiles, row statistics, mask words
   static constexpr int LDS_BYTES = 2 * STAGE_BYTES;                // double buffer
 };
 
@@ -134,6 +137,18 @@ __device__ __forceinline__ unsigned int pack_half2(float a, float b) {
   return __builtin_bit_cast(unsigned int, h);
 }
 
+// scores of unset mask elements become -inf; mw: the 64 mask bits of this lane's row, already
+// shifted right by 4 g, so that bit 8(i/4) + i%4 (+ 32 for the second block) belongs to register i
+__device__ __forceinline__ void mask_scores(floatx16& s0, floatx16& s1, unsigned long long mw) {
+  const unsigned lo = (unsigned)mw, hi = (unsigned)(mw >> 32);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const unsigned bit = 1u << (8 * (i / 4) + (i % 4));
+    s0[i] = (lo & bit) ? s0[i] : -INFINITY;
+    s1[i] = (hi & bit) ? s1[i] : -INFINITY;
+  }
+}
+
 __device__ __forceinline__ floatx16 zero16() {
   floatx16 z;
 #pragma unroll
@@ -156,9 +171,9 @@ __device__ __forceinline__ void head_and_block(int L, int BH, int nb, int& bh, i
 // ---------------------------------------------------------------------------------------
 // dQ: workgroup = row block m, wavefront wv owns queries 64m + 32wv + ln
 // ---------------------------------------------------------------------------------------
-template <int D, bool BF16>
+template <int D, bool BF16, bool EW>
 __global__ __launch_bounds__(128) void dq_kernel(const BwdParams prm) {
-  using C = BwdCfg<D>;
+  using C = BwdCfg<D, EW>;
   constexpr int KS = D / 16, DB = D / 32;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -182,6 +197,9 @@ __global__ __launch_bounds__(128) void dq_kernel(const BwdParams prm) {
     half_tile_load_async<D>(kg + (int64_t)cb * 64 * prm.ks[2], prm.ks[2], wv, lane, lds_addr + stage * C::STAGE_BYTES);
     half_tile_load_async<D>(vg + (int64_t)cb * 64 * prm.vs[2], prm.vs[2], wv, lane,
                             lds_addr + stage * C::STAGE_BYTES + C::TILE_BYTES);
+    if constexpr (EW)   // the tile's 64 mask words, 256 bytes per wavefront
+      stat_load_async(reinterpret_cast<const float*>(prm.bits_rows + (int64_t)t * 64) + wv * 64, lane,
+                      lds_addr + stage * C::STAGE_BYTES + 2 * C::TILE_BYTES + C::STAT_BYTES + wv * 256);
   };
   if (t0 < t1) issue(t0, 0);
 
@@ -194,7 +212,9 @@ __global__ __launch_bounds__(128) void dq_kernel(const BwdParams prm) {
     qfr[s] = *reinterpret_cast<const uintx4*>(qp + 16 * s + 8 * g);
     dofr[s] = *reinterpret_cast<const uintx4*>(gp + 16 * s + 8 * g);
   }
-  const float lse2 = prm.lse[(int64_t)bh * prm.N + qrow] * kLog2e;
+  // a query without any unmasked key has lse = -inf: every P of its row must come out as 0
+  const float lse_q = prm.lse[(int64_t)bh * prm.N + qrow];
+  const float lse2 = EW && lse_q == -INFINITY ? INFINITY : lse_q * kLog2e;
   const float dlt = prm.delta[(int64_t)bh * prm.N + qrow];
   // compiler-visible vmcnt(0): everything above has arrived, no vector-memory waits in the loop
   __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -234,6 +254,11 @@ __global__ __launch_bounds__(128) void dq_kernel(const BwdParams prm) {
         dpacc[kb] = mfma_qk<BF16>(fv[kb][s], dofr[s], dpacc[kb]);   // dP^T = V dO^T
       }
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (EW) {
+      const unsigned long long mw = *reinterpret_cast<const unsigned long long*>(
+          vt + C::TILE_BYTES + C::STAT_BYTES + (32 * wv + ln) * 8) >> (4 * g);
+      mask_scores(sacc[0], sacc[1], mw);
+    }
     // K^T fragments of the second product, read under the exponentials below
     uintx4 fkt[4][DB];
 #pragma unroll
@@ -272,9 +297,9 @@ __global__ __launch_bounds__(128) void dq_kernel(const BwdParams prm) {
 // ---------------------------------------------------------------------------------------
 // dK, dV: workgroup = column block n, wavefront wv owns keys 64n + 32wv + ln
 // ---------------------------------------------------------------------------------------
-template <int D, bool BF16>
+template <int D, bool BF16, bool EW>
 __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
-  using C = BwdCfg<D>;
+  using C = BwdCfg<D, EW>;
   constexpr int KS = D / 16, DB = D / 32;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -300,6 +325,9 @@ __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
     half_tile_load_async<D>(qg + (int64_t)rb * 64 * prm.qs[2], prm.qs[2], wv, lane, sa);
     half_tile_load_async<D>(gg + (int64_t)rb * 64 * prm.dos[2], prm.dos[2], wv, lane, sa + C::TILE_BYTES);
     stat_load_async((wv == 0 ? lse_h : dlt_h) + rb * 64, lane, sa + 2 * C::TILE_BYTES + wv * 256);
+    if constexpr (EW)   // the tile's 64 mask words (one per key, bit = query), 256 bytes per wavefront
+      stat_load_async(reinterpret_cast<const float*>(prm.bits_cols + (int64_t)t * 64) + wv * 64, lane,
+                      sa + 2 * C::TILE_BYTES + C::STAT_BYTES + wv * 256);
   };
   if (t0 < t1) issue(t0, 0);
 
@@ -350,6 +378,11 @@ __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
         dpacc[qb] = mfma_qk<BF16>(fg[qb][s], vfr[s], dpacc[qb]);    // dP = dO V^T
       }
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (EW) {
+      const unsigned long long mw = *reinterpret_cast<const unsigned long long*>(
+          gt + C::TILE_BYTES + C::STAT_BYTES + (32 * wv + ln) * 8) >> (4 * g);
+      mask_scores(sacc[0], sacc[1], mw);
+    }
     // dO^T and Q^T fragments of the second products, read under the exponentials below
     uintx4 fgt[4][DB], fqt[4][DB];
 #pragma unroll
@@ -373,7 +406,9 @@ __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
         float p[4], ds[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[qb][i0 + e], qk_scale, -l4[e] * kLog2e));
+          // (a query without any unmasked key has lse = -inf: its P must come out as 0)
+          const float nl = EW && l4[e] == -INFINITY ? -INFINITY : -l4[e] * kLog2e;
+          p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[qb][i0 + e], qk_scale, nl));
           ds[e] = p[e] * (dpacc[qb][i0 + e] - d4[e]);
         }
         pf[ts][2 * jh] = pack_half2(p[0], p[1]);   pf[ts][2 * jh + 1] = pack_half2(p[2], p[3]);
@@ -411,14 +446,14 @@ size_t bwd_workspace_bytes(int B, int H, int N, int D) {
   return (size_t)B * H * N * sizeof(float);   // delta
 }
 
-template <int D, bool BF16>
+template <int D, bool BF16, bool EW>
 static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
-  using C = BwdCfg<D>;
+  using C = BwdCfg<D, EW>;
   static bool configured = false;   // raising the dynamic LDS limit is idempotent
   if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dq_kernel<D, BF16>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dq_kernel<D, BF16, EW>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv_kernel<D, BF16>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv_kernel<D, BF16, EW>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
     configured = true;
   }
@@ -426,18 +461,20 @@ static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
   constexpr int RPB = 256 / (D / 8);
   hipLaunchKernelGGL((delta_kernel<D, BF16>), dim3((prm.N + RPB - 1) / RPB, BH), dim3(256), 0, st, prm);
   const int grid = ((BH + 7) / 8) * 8 * prm.nb;   // heads in groups of 8, the last group padded
-  hipLaunchKernelGGL((dq_kernel<D, BF16>), dim3(grid), dim3(128), C::LDS_BYTES, st, prm);
-  hipLaunchKernelGGL((dkdv_kernel<D, BF16>), dim3(grid), dim3(128), C::LDS_BYTES, st, prm);
+  hipLaunchKernelGGL((dq_kernel<D, BF16, EW>), dim3(grid), dim3(128), C::LDS_BYTES, st, prm);
+  hipLaunchKernelGGL((dkdv_kernel<D, BF16, EW>), dim3(grid), dim3(128), C::LDS_BYTES, st, prm);
 }
 
 int launch_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
                const float* lse, void* dq, void* dk, void* dv, const int32_t* row_ptr,
                const int32_t* col_idx, const int32_t* col_ptr, const int32_t* row_idx,
+               const uint64_t* bits_rows, const uint64_t* bits_cols,
                const AttnShape& s, void* ws, hipStream_t st) {
   BwdParams prm;
   prm.q = q; prm.k = k; prm.v = v; prm.o = o; prm.d_o = d_o; prm.lse = lse; prm.delta = (float*)ws;
   prm.dq = dq; prm.dk = dk; prm.dv = dv;
   prm.row_ptr = row_ptr; prm.col_idx = col_idx; prm.col_ptr = col_ptr; prm.row_idx = row_idx;
+  prm.bits_rows = (const unsigned long long*)bits_rows; prm.bits_cols = (const unsigned long long*)bits_cols;
   prm.B = s.B; prm.H = s.H; prm.N = s.N; prm.nb = s.N / 64; prm.Bm = s.Bm; prm.Hm = s.Hm;
   prm.out_f32 = s.out_dtype == BSATTN_F32;
   prm.sm_scale = s.sm_scale;
@@ -446,10 +483,17 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* o, const
     prm.qs[i] = s.qs[i]; prm.ks[i] = s.ks[i]; prm.vs[i] = s.vs[i]; prm.os[i] = s.os[i]; prm.dos[i] = s.dos[i];
   }
   const bool bf = s.dtype == BSATTN_BF16;
-  if (s.D == 64 && !bf) launch_bwd_t<64, false>(prm, st);
-  else if (s.D == 64 && bf) launch_bwd_t<64, true>(prm, st);
-  else if (s.D == 128 && !bf) launch_bwd_t<128, false>(prm, st);
-  else launch_bwd_t<128, true>(prm, st);
+  if (bits_rows == nullptr) {
+    if (s.D == 64 && !bf) launch_bwd_t<64, false, false>(prm, st);
+    else if (s.D == 64 && bf) launch_bwd_t<64, true, false>(prm, st);
+    else if (s.D == 128 && !bf) launch_bwd_t<128, false, false>(prm, st);
+    else launch_bwd_t<128, true, false>(prm, st);
+  } else {   // elementwise mask
+    if (s.D == 64 && !bf) launch_bwd_t<64, false, true>(prm, st);
+    else if (s.D == 64 && bf) launch_bwd_t<64, true, true>(prm, st);
+    else if (s.D == 128 && !bf) launch_bwd_t<128, false, true>(prm, st);
+    else launch_bwd_t<128, true, true>(prm, st);
+  }
   return launch_status();
 }
 

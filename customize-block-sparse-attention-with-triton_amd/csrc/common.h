@@ -37,6 +37,7 @@ size_t bwd_workspace_bytes(int B, int H, int N, int D);
 int launch_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
                const float* lse, void* dq, void* dk, void* dv, const int32_t* row_ptr,
                const int32_t* col_idx, const int32_t* col_ptr, const int32_t* row_idx,
+               const uint64_t* bits_rows, const uint64_t* bits_cols,
                const AttnShape& s, void* ws, hipStream_t st);
 
 // reorder.hip

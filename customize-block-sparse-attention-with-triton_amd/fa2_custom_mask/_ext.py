@@ -31,6 +31,7 @@ _SIGNATURES = {
                                 _p, _p, _p, _p, _p, ctypes.c_size_t, _p], _i),
     "bsattn_bwd_workspace": ([_i, _i, _i, _i, ctypes.POINTER(ctypes.c_size_t)], _i),
     "bsattn_bwd": ([_p] * 13 + [_i] * 8 + [_f] + [_p] * 5 + [_p, ctypes.c_size_t, _p], _i),
+    "bsattn_bwd_elementwise": ([_p] * 15 + [_i] * 8 + [_f] + [_p] * 5 + [_p, ctypes.c_size_t, _p], _i),
     "bsattn_reorder": ([_p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p], _i),
     "bsattn_mfma_rate_probe": ([_p, _i, _p, _p, _p], _i),
 }

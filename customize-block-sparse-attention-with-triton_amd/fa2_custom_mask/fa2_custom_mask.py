@@ -120,14 +120,18 @@ def _backward(q, k, v, o, do, lse, lists, lists_t, sm_scale, out_dtype):
     dv = torch.empty_like(dq)
     wsb = _ext.bwd_workspace(B, H, N, D)
     ws = torch.empty(wsb, dtype=torch.uint8, device=q.device)
-    rc = _ext.lib().bsattn_bwd(
-        q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(), lse.data_ptr(),
-        dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
-        lists.row_ptr.data_ptr(), lists.col_idx.data_ptr(), lists_t.row_ptr.data_ptr(),
-        lists_t.col_idx.data_ptr(), lists.Bm, lists.Hm, B, H, N, D,
-        _ext.dtype_code(q.dtype), _ext.dtype_code(out_dtype), float(sm_scale),
-        _ext.strides4(q), _ext.strides4(k), _ext.strides4(v), _ext.strides4(o), _ext.strides4(do),
-        ws.data_ptr(), wsb, _ext.current_stream(q.device))
+    tensors = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(), lse.data_ptr(),
+               dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+               lists.row_ptr.data_ptr(), lists.col_idx.data_ptr(), lists_t.row_ptr.data_ptr(),
+               lists_t.col_idx.data_ptr())
+    common = (lists.Bm, lists.Hm, B, H, N, D,
+              _ext.dtype_code(q.dtype), _ext.dtype_code(out_dtype), float(sm_scale),
+              _ext.strides4(q), _ext.strides4(k), _ext.strides4(v), _ext.strides4(o), _ext.strides4(do),
+              ws.data_ptr(), wsb, _ext.current_stream(q.device))
+    if lists.bits is None:
+        rc = _ext.lib().bsattn_bwd(*tensors, *common)
+    else:                                      # elementwise mask
+        rc = _ext.lib().bsattn_bwd_elementwise(*tensors, lists.bits.data_ptr(), lists_t.bits.data_ptr(), *common)
     _ext.check(rc, "bsattn_bwd")
     return dq, dk, dv
 

@@ -161,6 +161,23 @@ int bsattn_bwd(const void* q, const void* k, const void* v, const void* o, const
                void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------
+ * Backward with an elementwise mask: as bsattn_bwd, with P = 0 at unset elements (the
+ * zeroing fa2_bwd.py:59-62,119-123 intends).  tile_bits_rows: words of the row lists
+ * (bsattn_pack_mask_tiles on row_ptr/col_idx), tile_bits_cols: words of the column lists
+ * (the same call on col_ptr/row_idx with the mask's row and column strides swapped).
+ * Rows whose lse is -inf get zero gradients.
+ * ---------------------------------------------------------------------------------- */
+int bsattn_bwd_elementwise(const void* q, const void* k, const void* v, const void* o, const void* d_o,
+                           const float* lse, void* dq, void* dk, void* dv, const int32_t* row_ptr,
+                           const int32_t* col_idx, const int32_t* col_ptr, const int32_t* row_idx,
+                           const uint64_t* tile_bits_rows, const uint64_t* tile_bits_cols,
+                           int Bm, int Hm, int B, int H, int N, int D, int dtype, int out_dtype,
+                           float sm_scale, const int64_t* q_strides, const int64_t* k_strides,
+                           const int64_t* v_strides, const int64_t* o_strides,
+                           const int64_t* do_strides, void* workspace, size_t workspace_bytes,
+                           void* stream);
+
+/* ------------------------------------------------------------------------------------
  * Head-wise token reorder.  Replaces reorder_kernel / inv_reorder_kernel
  * (fa2_custom_mask/permute.py:5-58, 60-126) as launched from apply_head_wise_reorder /
  * apply_inv_reorder (fa2_custom_mask/functional.py:5-20, 46-62).

@@ -88,3 +88,42 @@ def test_tile_constant_elementwise_equals_block(dev):
     q, k, v = [x.to(dev) for x in make_qkv(1, 2, N, 64, torch.float16, 60)]
     assert same_up_to_rounding(fm.flash_attention_custom_mask(q, k, v, dense.to(dev), 0.125),
                                fm.flash_attention_custom_mask(q, k, v, block.to(dev), 0.125))
+
+
+@pytest.mark.parametrize("D,dtype", [(64, torch.float16), (128, torch.bfloat16)])
+def test_backward_elementwise(dev, D, dtype):
+    """dQ, dK, dV with elementwise masks (token-causal, and random with empty tiles, full tiles and
+    queries without keys) against the oracle's gradient of the naive masked softmax."""
+    import fa2_custom_mask as fm
+    g = torch.Generator().manual_seed(61)
+    N = 384
+    rnd = torch.rand(1, 2, N, N, generator=g) < 0.4
+    rnd[0, 0, :, 64:128] = False
+    rnd[0, 1, 128:192, :] = True
+    rnd[0, 1, 7, :] = False
+    rnd[0, 0, 320:, :] = False
+    for mask in (token_causal(N), rnd):
+        H = 2
+        q, k, v, do = make_qkv(1, H, N, D, dtype, 62, n=4)
+        sc = 1.0 / np.sqrt(D)
+        dq_r, dk_r, dv_r, _ = orc.attention_backward(f32(q), f32(k), f32(v), mask.numpy(), sc, f32(do))
+        o, lse, dq, dk, dv = fm.attention_forward_backward(q.to(dev), k.to(dev), v.to(dev), mask.to(dev), sc,
+                                                           do.to(dev), out_fp32=True)
+        torch.cuda.synchronize()
+        for name, got, ref in (("dq", dq, dq_r), ("dk", dk, dk_r), ("dv", dv, dv_r)):
+            ma, rl = errors(got, ref)
+            print("%s D%d %s: max-abs %.3e rel-L2 %.3e" % (name, D, dtype, ma, rl))
+            assert np.isfinite(f32(got)).all()
+            assert ma <= MAXABS[dtype] and rl <= 1e-3
+
+
+def test_autograd_with_elementwise_mask(dev):
+    import fa2_custom_mask as fm
+    N = 256
+    mask = token_causal(N)
+    q, k, v, do = make_qkv(1, 1, N, 64, torch.float16, 63, n=4)
+    dq_r, dk_r, dv_r, _ = orc.attention_backward(f32(q), f32(k), f32(v), mask.numpy(), 0.125, f32(do))
+    qd, kd, vd = [x.to(dev).requires_grad_(True) for x in (q, k, v)]
+    fm.flash_attention_custom_mask(qd, kd, vd, mask.to(dev), 0.125).backward(do.to(dev))
+    for got, ref in ((qd.grad, dq_r), (kd.grad, dk_r), (vd.grad, dv_r)):
+        assert errors(got, ref)[0] <= 2e-2
