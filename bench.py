@@ -69,6 +69,33 @@ def fwd_bwd_c5(torch, dev, fm, steps, warmup):
             "note": "times include the per-call output/workspace allocation of the host wrapper"}
 
 
+def elementwise_case(torch, dev, fm, q, k, v, sm_scale):
+    """Token-level causal mask [1,1,N,N] at the headline shape: every diagonal tile is partly set.
+    Forward time with the packed mask words applied, and the time of the elementwise preprocessing
+    (reduce + lists + pack of the 307.5 MB mask)."""
+    from fa2_custom_mask import utils
+    mask = torch.ones(N, N, dtype=torch.bool, device=dev).tril_().reshape(1, 1, N, N)
+    lists = utils.mask_to_lists(mask, N)
+    tiles = int(lists.counts[1])
+    o, _ = fm.fa2_custom_mask._forward(q, k, v, lists, sm_scale, torch.float16, True)
+    tf = event_times(lambda: fm.fa2_custom_mask._forward(q, k, v, lists, sm_scale, torch.float16, False), 20, 3, torch)
+
+    def prep():
+        utils.lists_cache.clear()
+        utils.mask_to_lists(mask, N)
+    tp = event_times(prep, 10, 2, torch)
+    # parity spot check against torch on the first 128 and last 64 queries
+    rows = torch.cat([torch.arange(128), torch.arange(N - 64, N)]).to(dev)
+    s = (q[0, 0, rows].float() @ k[0, 0].float().T) * sm_scale
+    s = s.masked_fill(~mask[0, 0, rows], float("-inf"))
+    ref = torch.softmax(s, -1) @ v[0, 0].float()
+    err = float((o[0, 0, rows].float() - ref).abs().max())
+    mf = tf[len(tf) // 2]
+    return {"workload": "token-level causal mask, N=17536 D=64 fp16", "kept_tiles": tiles,
+            "fwd_ms": round(mf, 5), "fwd_tflops_on_kept_tiles": round(tile_flops(tiles) / mf / 1e9, 1),
+            "preprocess_ms": round(tp[len(tp) // 2], 5), "max_abs_vs_torch_fp32": err}
+
+
 def mfma_ceiling(torch, dev, iters=8192, launches=10):
     """Sustained fp16 MFMA rate (TFLOP/s) of bsattn_mfma_rate_probe for two operand patterns."""
     import ctypes
@@ -214,6 +241,7 @@ def main():
                             "block_mask_ms": round(ts_b[len(ts_b) // 2], 5)},
         "parity_max_abs_vs_oracle": parity,
         "fwd_bwd_configs4": fwd_bwd_c5(torch, dev, fm, 20, 3),
+        "elementwise_mask": elementwise_case(torch, dev, fm, qd, kd, vd, sm_scale),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
                      "kernel": "fwd_kernel<64,false,false> (one bsattn_fwd call)",
