@@ -117,10 +117,12 @@ __global__ __launch_bounds__(256) void fill_rows_kernel(const uint8_t* __restric
 // Elementwise masks: the 64 x 64 bools of every kept tile packed into 64 words of 64 bits
 // (word r = row r of the tile, bit c = column c), plus a flag per kept tile saying whether the
 // tile is only partly set.  Slot t of `bits` / `partial` belongs to entry t of the kept-tile
-// list.  One workgroup per mask row block, its wavefronts striding over the row block's kept
-// tiles; lane l packs row l of the tile.  With the row and column strides of the mask and the
+// list.  PACK_SPLIT workgroups of 4 wavefronts per mask row block, their wavefronts striding over
+// the row block's kept tiles (a wavefront has one tile's loads in flight at a time, so the
+// kernel lives on the number of wavefronts); lane l packs row l of the tile.  With the row and column strides of the mask and the
 // lists both transposed, the words describe the columns (what the dK/dV pass needs).
 // ---------------------------------------------------------------------------------------
+constexpr int PACK_SPLIT = 8;
 __global__ __launch_bounds__(256) void pack_tiles_kernel(const uint8_t* __restrict__ dense, int nb, int H,
                                                          int64_t sb, int64_t sh, int64_t sm, int64_t sn,
                                                          const int32_t* __restrict__ row_ptr,
@@ -128,11 +130,11 @@ __global__ __launch_bounds__(256) void pack_tiles_kernel(const uint8_t* __restri
                                                          uint8_t* __restrict__ partial,
                                                          unsigned long long* __restrict__ bits) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int rb = blockIdx.x, bh = blockIdx.y;
+  const int rb = blockIdx.x / PACK_SPLIT, sub = blockIdx.x % PACK_SPLIT, bh = blockIdx.y;
   const int32_t* rp = row_ptr + (int64_t)bh * nb;
   const int t0 = rp[rb], t1 = rp[rb + 1];
   const uint8_t* rowp = dense + (bh / H) * sb + (bh % H) * sh + ((int64_t)rb * 64 + lane) * sm;
-  for (int t = t0 + wave; t < t1; t += 4) {
+  for (int t = t0 + sub * 4 + wave; t < t1; t += 4 * PACK_SPLIT) {
     const uint8_t* p = rowp + (int64_t)col_idx[t] * 64 * sn;
     unsigned long long word = 0ull;
     if (sn == 1) {
@@ -178,7 +180,7 @@ int launch_block_mask_to_lists(const uint8_t* block, int Bm, int Hm, int nb, int
 int launch_pack_tiles(const uint8_t* dense, int Bm, int Hm, int nb, int64_t sb, int64_t sh, int64_t sm,
                       int64_t sn, const int32_t* row_ptr, const int32_t* col_idx, uint8_t* partial,
                       unsigned long long* bits, hipStream_t st) {
-  hipLaunchKernelGGL(pack_tiles_kernel, dim3(nb, Bm * Hm), dim3(256), 0, st, dense, nb, Hm, sb, sh, sm, sn,
+  hipLaunchKernelGGL(pack_tiles_kernel, dim3(nb * PACK_SPLIT, Bm * Hm), dim3(256), 0, st, dense, nb, Hm, sb, sh, sm, sn,
                      row_ptr, col_idx, partial, bits);
   return launch_status();
 }
