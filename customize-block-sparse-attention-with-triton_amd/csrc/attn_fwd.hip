@@ -432,6 +432,32 @@ void fwd_kernel(const FwdParams prm) {
     __builtin_amdgcn_sched_barrier(0);
   };
 
+  // Number of entries r in [0, nb] with rp[r] <= x, for two values of x at once.  The row pointers
+  // ascend, so this is a search; it is done in two rounds of one load per lane (64 evenly spaced
+  // entries, then the entries between two of them) instead of a chain of dependent scalar loads.
+  auto count_le2 = [&](int x0, int x1, int& c0, int& c1) {
+    const int32_t* rpg_ = prm.row_ptr + (int64_t)mh * nb;
+    const int step = (nb + 64) / 64;
+    if (step > 64) {     // very long sequences: plain binary searches
+      int lo = -1, hi = nb + 1;
+      while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (rp[mid] <= x0) lo = mid; else hi = mid; }
+      c0 = hi;
+      lo = -1; hi = nb + 1;
+      while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (rp[mid] <= x1) lo = mid; else hi = mid; }
+      c1 = hi;
+      return;
+    }
+    const int i1 = lane * step;
+    const int v1 = i1 <= nb ? rpg_[i1] : 0x7fffffff;
+    const int a0 = __builtin_popcountll(__ballot(v1 <= x0)), a1 = __builtin_popcountll(__ballot(v1 <= x1));
+    const int b0 = (a0 > 0 ? a0 - 1 : 0) * step, b1 = (a1 > 0 ? a1 - 1 : 0) * step;
+    const int j0 = b0 + lane, j1 = b1 + lane;
+    const int w0 = lane < step && j0 <= nb ? rpg_[j0] : 0x7fffffff;
+    const int w1 = lane < step && j1 <= nb ? rpg_[j1] : 0x7fffffff;
+    c0 = a0 > 0 ? b0 + __builtin_popcountll(__ballot(w0 <= x0)) : 0;
+    c1 = a1 > 0 ? b1 + __builtin_popcountll(__ballot(w1 <= x1)) : 0;
+  };
+
   int* ctr = reinterpret_cast<int*>(ml + NW * 2 * 64);
   int* lcols = ctr + 16;
   // The column indices of the range are staged in LDS: a scalar load per tile would put its whole
@@ -529,12 +555,10 @@ void fwd_kernel(const FwdParams prm) {
     // alone and writes its result directly: no merge, no partials.
     int r_lo, r_hi;
     {
-      int lo = -1, hi = nb;   // smallest r with rp[r] >= g0
-      while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (rp[mid] >= g0) hi = mid; else lo = mid; }
-      r_lo = hi;
-      lo = -1; hi = nb;       // smallest r with rp[r] >= g1
-      while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (rp[mid] >= g1) hi = mid; else lo = mid; }
-      r_hi = hi;
+      // smallest r with rp[r] >= g = number of r with rp[r] <= g - 1 (capped at nb)
+      count_le2(g0 - 1, g1 - 1, r_lo, r_hi);
+      r_lo = r_lo < nb ? r_lo : nb;
+      r_hi = r_hi < nb ? r_hi : nb;
       if (wg >= hs.Peff - 1) r_hi = nb;    // trailing row blocks without kept tiles
       if (wg == 0) r_lo = 0;               // leading ones
     }
@@ -556,9 +580,9 @@ void fwd_kernel(const FwdParams prm) {
     // first row block of the range: largest r with rp[r] <= g0 < rp[r+1]
     int r;
     {
-      int lo = 0, hi = nb;  // invariant: rp[lo] <= g0 < rp[hi]
-      while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (rp[mid] <= g0) lo = mid; else hi = mid; }
-      r = lo;
+      int c0, c1;
+      count_le2(g0, g0, c0, c1);
+      r = c0 - 1;
     }
     stage_cols(g0, g1);
     if (threadIdx.x == 0) { ctr[0] = g0 + 2 * NW; ctr[3] = 0; }
