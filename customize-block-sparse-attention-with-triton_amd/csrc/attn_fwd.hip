@@ -139,7 +139,7 @@ template <int D> struct FwdCfg {
   static constexpr int COLS_CAP = 2048;                     // column indices of the range kept in LDS
   static constexpr int BITS_OFF = NW * WAVE_LDS + ML_BYTES + COLS_CAP * 4;   // mask words of the current tile, 512 bytes per wavefront
   static constexpr int LDS_BYTES = BITS_OFF + NW * 512;
-  static constexpr int R = TILE_BYTES / 256;                // accumulator registers exchanged per round
+  static constexpr int R = WAVE_LDS / 256;                  // accumulator registers exchanged per round (K and V buffer)
   static constexpr int ROUNDS = D / R;
   static constexpr int QPW = (R / 4) / NW;                  // output quads per wavefront and round
   static constexpr int SHORT_ROW = 6 * NW;                  // row blocks up to this many tiles may go to one wavefront
@@ -575,8 +575,8 @@ void fwd_kernel(const FwdParams prm) {
     // tile `cur` and has already drawn its next one `nxt`, so that it can prefetch it.  Tiles are
     // drawn in list order, so a wavefront's tiles increase, and `cur >= seg_b` means "nothing left
     // for me in this row block".  kdone / vdone name the tile whose copy into this wavefront's
-    // K / V buffer has been issued; a V copy is held back across the merge of a row block, which
-    // borrows the V buffers.
+    // K / V buffer has been issued; no copy is issued across the merge of a row block, which
+    // borrows both buffers of every wavefront (one exchange round for the whole accumulator).
     // first row block of the range: largest r with rp[r] <= g0 < rp[r+1]
     int r;
     {
@@ -640,7 +640,8 @@ void fwd_kernel(const FwdParams prm) {
           // draw the tile after next; the value is picked up inside the tile
           int drawn = 0;
           if (lane == 0) drawn = atomicAdd(ctr, 1);
-          const bool has1 = nxt < g1, copy_v = nxt < seg_b;
+          // the next tile is only prefetched inside the row block: the merge at its end borrows both buffers
+          const bool has1 = nxt < seg_b, copy_v = has1;
           int nn = 0, cb_nn_v = 0;
           tile(has1, cb_nxt & COL_MASK, nxt, copy_v, (cx >> 30) != 0, [&] {
             nn = __builtin_amdgcn_readfirstlane(drawn);
@@ -691,7 +692,7 @@ void fwd_kernel(const FwdParams prm) {
           {
             // every wavefront writes (one without tiles of this row block holds zeros), 4 bytes per
             // lane and instruction: wider LDS writes are much slower per byte on this hardware
-            float* own = reinterpret_cast<float*>(lds_v);
+            float* own = reinterpret_cast<float*>(lds_k);
 #pragma unroll
             for (int e = 0; e < C::R; ++e) {
               const int idx = rd * C::R + e;
@@ -724,7 +725,7 @@ void fwd_kernel(const FwdParams prm) {
             float x[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int pw = 0; pw < NW; ++pw) {
-              const float* src = reinterpret_cast<const float*>(lds + pw * C::WAVE_LDS + C::TILE_BYTES);
+              const float* src = reinterpret_cast<const float*>(lds + pw * C::WAVE_LDS);
 #pragma unroll
               for (int e = 0; e < 4; ++e) x[e] += wgt[pw][qb] * src[(4 * quad + e) * 64 + lane];
             }
