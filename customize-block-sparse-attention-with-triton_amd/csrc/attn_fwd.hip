@@ -27,96 +27,10 @@
 #include <chrono>
 #include "common.h"
 #include "fwd_split.h"
+#include "fwd_tile.h"
 #include "kernel_util.h"
 
 namespace bsattn {
-
-struct FwdParams {
-  const void* q; const void* k; const void* v; void* o; float* lse;
-  const int32_t* row_ptr; const int32_t* col_idx;
-  const unsigned char* tile_partial;        // elementwise masks: per kept tile, 1 = only partly set
-  const unsigned long long* tile_bits;      // ... and its 64 row words (bit c = column c)
-  float* ws;                       // partial slots of row blocks shared between workgroups
-  unsigned long long* flags;       // one per slot: holds `epoch` once the slot's part is complete
-  unsigned long long epoch;        // distinguishes this launch's flags from stale contents
-  int B, H, N, nb, Bm, Hm, W;   // W: workgroups per head
-  int first_ids;                // workgroups with a linear id below this are the first on their compute unit
-  int out_f32;
-  float qk_scale;  // sm_scale * log2(e)
-  int64_t qs[3], ks[3], vs[3], os[3];
-};
-
-// P = exp2(score - m) for the 2 x 16 scores one lane holds of one query (key blocks s0, s1),
-// rounded to fp16 and packed as the operand fragments pf[0..3][qb] of the second product.
-// Returns l + the row sum of the rounded P over this lane's keys.  With FOLD the scores
-// already are "scaled score - m".
-template <bool FOLD>
-__device__ __forceinline__ float softmax_tile(const floatx16& s0, const floatx16& s1, float qk_scale, float m,
-                                              float l, uintx4 (&pf)[4][2], int qb) {
-  const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
-#pragma unroll
-  for (int ts = 0; ts < 4; ++ts) {
-#pragma unroll
-    for (int jj = 0; jj < 4; ++jj) {
-      const int i = 8 * (ts & 1) + 2 * jj;
-      const float x0 = ts < 2 ? s0[i] : s1[i], x1 = ts < 2 ? s0[i + 1] : s1[i + 1];
-      const float p0 = __builtin_amdgcn_exp2f(FOLD ? x0 : __builtin_fmaf(x0, qk_scale, -m));
-      const float p1 = __builtin_amdgcn_exp2f(FOLD ? x1 : __builtin_fmaf(x1, qk_scale, -m));
-      const half2v hp = {(_Float16)p0, (_Float16)p1};
-      l = __builtin_amdgcn_fdot2(hp, ones, l, false);
-      pf[ts][qb][jj] = __builtin_bit_cast(unsigned int, hp);
-    }
-  }
-  return l;
-}
-
-__device__ __forceinline__ void* out_base(const FwdParams& prm, int b, int h) {
-  const int64_t off = b * prm.os[0] + h * prm.os[1];
-  return prm.out_f32 ? (void*)((float*)prm.o + off) : (void*)((unsigned short*)prm.o + off);
-}
-
-// Rare path of the softmax: re-centre the reference exponent of one query block on the row
-// maximum of the current tile and redo the tile's numerators.
-// With elementwise masks (EW) a query may have had nothing but masked keys so far (l == 0, or the
-// whole tile masked: maximum -inf): such a lane takes the tile's maximum as its first reference.
-template <int DB, bool FOLD, bool EW>
-__device__ __forceinline__ void recentre(floatx16& s0, floatx16& s1, floatx16 (&oacc)[DB][2], int qb, float qk_scale,
-                                      float& m, float& l, uintx4& mfrag, bool fresh, int g) {
-  float mx = max3f(s0[0], s0[1], s0[2]);
-#pragma unroll
-  for (int i = 3; i < 15; i += 2) mx = max3f(mx, s0[i], s0[i + 1]);
-  mx = max3f(mx, s0[15], s1[0]);
-#pragma unroll
-  for (int i = 1; i < 15; i += 2) mx = max3f(mx, s1[i], s1[i + 1]);
-  mx = xhalf_max(fmaxf(mx, s1[15]));
-  // exponent of the largest entry relative to the current reference
-  const float smax = FOLD ? mx : __builtin_fmaf(mx, qk_scale, -m);
-  float delta = fresh ? smax : fmaxf(smax, 0.f);
-  bool nomass = false;
-  if constexpr (EW) {
-    nomass = !fresh && l == 0.f;
-    if (nomass) delta = smax;
-    if (smax == -INFINITY) delta = 0.f;
-  }
-  m += delta;
-  if (!fresh) {
-    const float alpha = nomass ? 1.0f : __builtin_amdgcn_exp2f(-delta);
-    l *= alpha;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) oacc[db][qb][i] *= alpha;
-  }
-  if constexpr (FOLD) {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) { s0[i] -= delta; s1[i] -= delta; }
-    const _Float16 hi = (_Float16)(-m);
-    const _Float16 lo = (_Float16)(-m - (float)hi);
-    const half2v hl = {hi, lo};
-    mfrag[0] = g == 0 ? __builtin_bit_cast(unsigned int, hl) : 0u;
-  }
-}
-
 
 // Partial results cross workgroups (and the L2 slices of different XCDs) inside one launch:
 // they are written and read with device-scope accesses, which go to the point of coherence.
@@ -884,6 +798,17 @@ size_t fwd_workspace_bytes(int B, int H, int N, int D) {
   return slots_bytes(B, H, W, D) + (size_t)B * H * W * sizeof(unsigned long long);
 }
 
+void launch_fwd_pair(const FwdParams& prm, int dt, bool elementwise, hipStream_t st);   // attn_fwd_pair.hip
+// D = 128 with enough row blocks in the launch to fill the chip goes to the kernel that gives each
+// row block to one wavefront pair (two wavefronts per SIMD, no merges between workgroups).  With
+// fewer row blocks its critical path is the longest row, which the host cannot see (the lists
+// stay on the device): from two row blocks per compute unit on it won in every measured case,
+// from one on only when rows are short (at most 32 tiles).
+static bool use_pair_kernel(int64_t row_blocks, int nb) {
+  const int64_t cus = compute_units();
+  return row_blocks >= 2 * cus || (row_blocks >= cus && nb <= 32);
+}
+
 // With few row blocks per workgroup all wavefronts of a workgroup share one row block at a time
 // (K and V tiles are spread over them and the results merged); with many (>= 8 per workgroup) each
 // wavefront takes whole row blocks, which needs no merge and no second kernel.
@@ -925,6 +850,10 @@ int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
   for (int i = 0; i < 3; ++i) { prm.qs[i] = s.qs[i]; prm.ks[i] = s.ks[i]; prm.vs[i] = s.vs[i]; prm.os[i] = s.os[i]; }
   const bool bf = s.dtype == BSATTN_BF16;
   const int BH = s.B * s.H;
+  if (s.D == 128 && use_pair_kernel((int64_t)BH * prm.nb, prm.nb)) {
+    launch_fwd_pair(prm, bf ? 1 : 0, tile_bits != nullptr, st);
+    return launch_status();
+  }
   if (tile_bits == nullptr) {
     if (s.D == 64 && !bf) launch_fwd_t<64, false, false>(prm, BH, st);
     else if (s.D == 64 && bf) launch_fwd_t<64, true, false>(prm, BH, st);

@@ -1,0 +1,288 @@
+// Block-sparse FlashAttention-2 forward, head dimension 128, for launches with many row blocks.
+//
+// At D = 128 a wavefront that owns 64 queries needs all 512 registers of its SIMD, so the
+// general kernel (attn_fwd.hip) runs one wavefront per SIMD and is bound by instruction issue.
+// Here a row block belongs to a pair of wavefronts, 32 queries each (256 registers: two
+// wavefronts per SIMD), which share one K and one V tile buffer: a workgroup is one pair, four
+// workgroups fit a compute unit, and the grid has one workgroup per (head, row block) - the
+// hardware's dispatcher balances the load, no merge is ever needed.  Heads are taken in groups
+// of 8, head i of a group on XCD i (workgroups go to XCDs round-robin by linear id), so that the
+// row blocks resident on an XCD share one head's K and V in its L2; long row blocks of
+// block-causal masks come first.
+//
+// Tile arithmetic, softmax and layouts are those of attn_fwd.hip (fa2_custom_mask/fa2_fwd.py:146-196
+// of the reference), with a single block of 32 queries per wavefront.
+#include "common.h"
+#include "fwd_tile.h"
+#include "kernel_util.h"
+
+namespace bsattn {
+
+constexpr int PAIR_COLS_CAP = 1024;                               // column indices of the row block kept in LDS
+constexpr int PAIR_LDS_BYTES = 2 * 16384 + 512 + PAIR_COLS_CAP * 4;   // K tile, V tile, mask words, columns
+
+template <int DT, bool EW>
+__global__ __launch_bounds__(128, 2) void fwd_pair_kernel(const FwdParams prm) {
+  constexpr int D = 128, KS = D / 16, DB = D / 32, CPR = D / 8, ROWB = 2 * D, TILE_BYTES = 64 * ROWB;
+  constexpr bool BF16 = DT != 0;
+  constexpr bool FOLD = !BF16;
+  constexpr int HALF = CPR / 2;                  // copy instructions per wavefront and tile
+  constexpr int KOPS = HALF + (EW ? 1 : 0), VOPS = HALF;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+  const int lane = threadIdx.x & 63;
+  const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int ln = lane & 31, g = lane >> 5;
+  const int nb = prm.nb, BH = prm.B * prm.H;
+  // linear id -> (head, row block): groups of 8 heads, one head per XCD, long row blocks first
+  int bh, m;
+  {
+    const int L = blockIdx.x;
+    const int grp = L / (8 * nb), l = L - grp * 8 * nb;
+    const int hg = BH - 8 * grp < 8 ? BH - 8 * grp : 8;
+    bh = 8 * grp + l % hg;
+    m = nb - 1 - l / hg;
+    if (m < 0) return;                           // padding of an incomplete last group
+  }
+  const int b = bh / prm.H, h = bh % prm.H;
+  const int mh = (prm.Bm > 1 ? b : 0) * prm.Hm + (prm.Hm > 1 ? h : 0);
+  const cint_ptr_t rp = (cint_ptr_t)(uintptr_t)(prm.row_ptr + (int64_t)mh * nb);
+  const int t0 = rp[m], t1 = rp[m + 1];
+  void* obase = out_base(prm, b, h);
+  const int64_t qrow = (int64_t)m * 64 + 32 * w + ln;          // this lane's query
+  if (t0 == t1) {                                // no kept tile: O = 0, lse = -inf
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4)
+        store_out4<BF16>(obase, qrow * prm.os[2] + 32 * db + 8 * i4 + 4 * g, prm.out_f32, 0.f, 0.f, 0.f, 0.f);
+    if (prm.lse != nullptr && g == 0) prm.lse[(int64_t)bh * prm.N + qrow] = -INFINITY;
+    return;
+  }
+
+  unsigned char* lds_k = lds;
+  unsigned char* lds_v = lds + TILE_BYTES;
+  const unsigned long long* lds_bits = reinterpret_cast<const unsigned long long*>(lds + 2 * TILE_BYTES);
+  int* lcols = reinterpret_cast<int*>(lds + 2 * TILE_BYTES + 512);
+  const unsigned lds_k_addr = (unsigned)(uintptr_t)(lds_ptr_t)lds;
+  const unsigned lds_v_addr = lds_k_addr + TILE_BYTES;
+  const unsigned lds_bits_addr = lds_k_addr + 2 * TILE_BYTES;
+
+  const unsigned short* qg = (const unsigned short*)prm.q + b * prm.qs[0] + h * prm.qs[1];
+  const unsigned short* kg = (const unsigned short*)prm.k + b * prm.ks[0] + h * prm.ks[1];
+  const unsigned short* vg = (const unsigned short*)prm.v + b * prm.vs[0] + h * prm.vs[1];
+  const float qk_scale = prm.qk_scale;
+
+  // column indices of the row block (EW: "partly set" in bit 30), staged once
+  const cint_ptr_t cols = (cint_ptr_t)(uintptr_t)prm.col_idx;
+  typedef const unsigned char __attribute__((address_space(4)))* cbyte_ptr_t;
+  auto flagged_col = [&](int t) {
+    int c = cols[t];
+    if constexpr (EW) c |= (int)((cbyte_ptr_t)(uintptr_t)prm.tile_partial)[t] << 30;
+    return c;
+  };
+  for (int i = threadIdx.x; i < t1 - t0 && i < PAIR_COLS_CAP; i += 128) {
+    int c = prm.col_idx[t0 + i];
+    if constexpr (EW) c |= (int)prm.tile_partial[t0 + i] << 30;
+    lcols[i] = c;
+  }
+  constexpr int COL_MASK = 0x3fffffff;
+  auto col_of = [&](int t) { return t - t0 < PAIR_COLS_CAP ? lcols[t - t0] : flagged_col(t); };
+
+  // asynchronous tile copies: copy instruction j covers tile rows [4j, 4j+4); this wavefront issues
+  // the instructions [HALF w, HALF (w+1)) of every tile (and 256 of the 512 bytes of mask words)
+  constexpr int RPI = 64 / CPR, KPER = 4;
+  unsigned koff[KPER], voff;
+  {
+    const int row0 = lane / CPR, ch = lane % CPR;
+#pragma unroll
+    for (int par = 0; par < KPER; ++par)
+      koff[par] = 2u * (unsigned)(row0 * (int)prm.ks[2] + ((ch ^ k_swz<D>(par * RPI + row0)) * 8));
+    voff = 2u * (unsigned)(row0 * (int)prm.vs[2] + ((ch ^ v_swz<D>(row0)) * 8));
+  }
+  auto k_copy = [&](int cb, int t) {
+    const unsigned short* tile = kg + (int64_t)cb * 64 * prm.ks[2];
+#pragma unroll
+    for (int jj = 0; jj < HALF; ++jj) {
+      const int j = w * HALF + jj;
+      tile_load_async_one(tile + (int64_t)j * RPI * prm.ks[2], koff[jj % KPER], lds_k_addr + j * 1024);
+    }
+    if constexpr (EW) {
+      const unsigned long long* src = prm.tile_bits + (int64_t)t * 64;
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, %2"
+                   :: "s"(lds_bits_addr + w * 256), "v"(4u * (unsigned)lane + 256u * w), "s"(src) : "memory", "m0");
+    }
+  };
+  auto v_copy = [&](int cb) {
+    const unsigned short* tile = vg + (int64_t)cb * 64 * prm.vs[2];
+#pragma unroll
+    for (int jj = 0; jj < HALF; ++jj) {
+      const int j = w * HALF + jj;
+      tile_load_async_one(tile + (int64_t)j * RPI * prm.vs[2], voff, lds_v_addr + j * 1024);
+    }
+  };
+  static_assert(HALF % KPER == 0, "the K swizzle pattern of a wavefront's instructions starts at phase 0");
+
+  // fragment addresses (as in attn_fwd.hip)
+  int kaddr[2][KS];
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const int row = 32 * kb + ln;
+      kaddr[kb][s] = row * ROWB + (((2 * s + g) ^ k_swz<D>(row)) * 16);
+    }
+  const int vblk = lane >> 4, vs_ = lane & 15;
+  const int vkey0 = 4 * (vblk >> 1) + (vs_ >> 2), vcol0 = 16 * (vblk & 1) + 4 * (vs_ & 3);
+  const uintx4 ones_frag = {g == 0 ? 0x3c003c00u : 0u, 0u, 0u, 0u};
+
+  // first tile's copies, then Q (this lane's query: second operand of S^T = K Q^T)
+  __syncthreads();                                  // lcols
+  int cx = __builtin_amdgcn_readfirstlane(col_of(t0));
+  k_copy(cx & COL_MASK, t0);
+  v_copy(cx & COL_MASK);
+  uintx4 qf[1][KS];
+  {
+    const unsigned short* qp = qg + qrow * prm.qs[2];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) qf[0][s] = *reinterpret_cast<const uintx4*>(qp + 16 * s + 8 * g);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0), visible to the compiler: Q and the first tiles
+  if constexpr (FOLD) {
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const uintx4 raw = qf[0][s];
+      const uintx4 scaled = {scale_half2(raw[0], qk_scale), scale_half2(raw[1], qk_scale),
+                             scale_half2(raw[2], qk_scale), scale_half2(raw[3], qk_scale)};
+      qf[0][s] = scaled;
+    }
+  }
+  floatx16 oacc[DB][2];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { oacc[db][0][i] = 0.f; oacc[db][1][i] = 0.f; }
+  float m_i = 0.f, l_i = 0.f;
+  uintx4 mfrag = {0u, 0u, 0u, 0u};
+  bool fresh = true;
+  __syncthreads();                                  // both halves of K(t0) and V(t0) are in LDS
+
+  for (int t = t0; t < t1; ++t) {
+    const bool has1 = t + 1 < t1;
+    const int cxn = has1 ? __builtin_amdgcn_readfirstlane(col_of(t + 1)) : 0;
+    const bool partial = EW && (cx >> 30) != 0;
+    // ---- K fragments (and the mask word of this lane's query) ----
+    uintx4 kfr[2][KS];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int s = 0; s < KS; ++s) kfr[kb][s] = *reinterpret_cast<const uintx4*>(lds_k + kaddr[kb][s]);
+    unsigned long long mw = 0ull;
+    if constexpr (EW) { if (partial) mw = lds_bits[32 * w + ln] >> (4 * g); }
+    lds_wait();
+    __syncthreads();                                // both wavefronts hold their K fragments: the K buffer is free
+    if (has1) k_copy(cxn & COL_MASK, t + 1);
+    // ---- S^T = K Q^T (- m when FOLD) ----
+    floatx16 s0, s1;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { s0[i] = 0.f; s1[i] = 0.f; }
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      s0 = mfma_qk<BF16>(kfr[0][s], qf[0][s], s0);
+      s1 = mfma_qk<BF16>(kfr[1][s], qf[0][s], s1);
+    }
+    if constexpr (FOLD) {
+      s0 = mfma_qk<BF16>(ones_frag, mfrag, s0);
+      s1 = mfma_qk<BF16>(ones_frag, mfrag, s1);
+    }
+    if constexpr (EW) {
+      if (partial) {
+        const unsigned lo = (unsigned)mw, hi = (unsigned)(mw >> 32);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const unsigned bit = 1u << (8 * (i / 4) + (i % 4));
+          s0[i] = (lo & bit) ? s0[i] : -INFINITY;
+          s1[i] = (hi & bit) ? s1[i] : -INFINITY;
+        }
+      }
+    }
+    // ---- softmax numerators ----
+    uintx4 pf[4][2];
+    float lnew = softmax_tile<FOLD>(s0, s1, qk_scale, m_i, l_i, pf, 0);
+    if (__any(fresh || (EW && l_i == 0.f) || !(lnew - l_i < 16384.0f))) {
+      recentre<DB, FOLD, EW>(s0, s1, oacc, 0, qk_scale, m_i, l_i, mfrag, fresh, g);
+      lnew = softmax_tile<FOLD>(s0, s1, qk_scale, m_i, l_i, pf, 0);
+    }
+    l_i = lnew;
+    fresh = false;
+    // ---- V^T fragments ----
+    if (has1) wait_vm<KOPS>(); else wait_vm<0>();   // this wavefront's half of V(t) has landed (K(t+1) may be in flight)
+    if (t > t0) __syncthreads();                    // ... and the other half (the first tile was waited for above)
+    uintx4 vfr[4][DB];
+#pragma unroll
+    for (int ts = 0; ts < 4; ++ts)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        uintx4 a;
+#pragma unroll
+        for (int jh = 0; jh < 2; ++jh) {
+          const int key = 16 * ts + 8 * jh + vkey0, col = 32 * db + vcol0;
+          const int addr = key * ROWB + (((col >> 3) ^ v_swz<D>(key)) * 16) + (col & 7) * 2;
+          const short4v rr = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (short4v __attribute__((address_space(3)))*)(lds_v + addr));
+          const uintx2 r2 = __builtin_bit_cast(uintx2, rr);
+          a[2 * jh] = r2[0]; a[2 * jh + 1] = r2[1];
+        }
+        if constexpr (BF16) a = bf16x8_to_f16x8(a);
+        vfr[ts][db] = a;
+      }
+    lds_wait();
+    __syncthreads();                                // both wavefronts hold their V fragments: the V buffer is free
+    if (has1) v_copy(cxn & COL_MASK);
+    // ---- O^T += V^T P^T ----
+#pragma unroll
+    for (int ts = 0; ts < 4; ++ts)
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+        oacc[db][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, vfr[ts][db]),
+                                                            __builtin_bit_cast(half8, pf[ts][0]), oacc[db][0], 0, 0, 0);
+    if (has1) {
+      wait_vm<VOPS>();                              // this wavefront's half of K(t+1) has landed (V(t+1) may be in flight)
+      __syncthreads();                              // ... and the other half
+    }
+    cx = cxn;
+  }
+
+  // ---- normalise and write ----
+  const float lsum = l_i + __shfl_xor(l_i, 32);
+  const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4)
+      store_out4<BF16>(obase, qrow * prm.os[2] + 32 * db + 8 * i4 + 4 * g, prm.out_f32, oacc[db][0][4 * i4] * inv,
+                       oacc[db][0][4 * i4 + 1] * inv, oacc[db][0][4 * i4 + 2] * inv, oacc[db][0][4 * i4 + 3] * inv);
+  if (prm.lse != nullptr && g == 0)
+    prm.lse[(int64_t)bh * prm.N + qrow] =
+        lsum > 0.f ? (m_i + __builtin_amdgcn_logf(lsum)) * 0.6931471805599453f : -INFINITY;
+}
+
+template <int DT, bool EW>
+static void launch_pair_t(const FwdParams& prm, hipStream_t st) {
+  static bool configured = false;
+  if (!configured) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_pair_kernel<DT, EW>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, PAIR_LDS_BYTES);
+    configured = true;
+  }
+  const int BH = prm.B * prm.H;
+  const int grid = ((BH + 7) / 8) * 8 * prm.nb;
+  hipLaunchKernelGGL((fwd_pair_kernel<DT, EW>), dim3(grid), dim3(128), PAIR_LDS_BYTES, st, prm);
+}
+
+// D = 128 only.  dt: 0 fp16, 1 bf16.
+void launch_fwd_pair(const FwdParams& prm, int dt, bool elementwise, hipStream_t st) {
+  if (!elementwise) { if (dt == 0) launch_pair_t<0, false>(prm, st); else launch_pair_t<1, false>(prm, st); }
+  else { if (dt == 0) launch_pair_t<0, true>(prm, st); else launch_pair_t<1, true>(prm, st); }
+}
+
+}  // namespace bsattn

@@ -79,6 +79,21 @@ def test_many_heads_elementwise(dev):
     check_forward(dev, 4, 64, N, 64, torch.float16, m, 58)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_many_heads_elementwise_d128(dev, dtype):
+    """D = 128 with many row blocks in the launch (one wavefront pair per row block) and partly set
+    tiles, queries without keys, an empty row block."""
+    g = torch.Generator().manual_seed(64)
+    N = 512
+    m = (torch.rand(1, 1, N, N, generator=g) < 0.6) & token_causal(N)
+    m[0, 0, 70, :] = False
+    m[0, 0, 128:192, :] = False
+    check_forward(dev, 4, 64, N, 128, dtype, m, 65)
+    m2 = torch.rand(4, 1, N, N, generator=g) < 0.3
+    m2[2, 0, :, :64] = False
+    check_forward(dev, 4, 64, N, 128, dtype, m2, 66)
+
+
 def test_tile_constant_elementwise_equals_block(dev):
     import fa2_custom_mask as fm
     from helpers import uniform_block_mask, same_up_to_rounding
