@@ -66,6 +66,15 @@ int bsattn_pack_mask_tiles(const uint8_t* dense, int Bm, int Hm, int N, int64_t 
                            (unsigned long long*)tile_bits, (hipStream_t)stream);
 }
 
+int bsattn_tail_mask_tiles(int Bm, int Hm, int nb, int valid_last, int transposed, const int32_t* row_ptr,
+                           const int32_t* col_idx, uint8_t* tile_partial, uint64_t* tile_bits, void* stream) {
+  if (row_ptr == nullptr || col_idx == nullptr || tile_partial == nullptr || tile_bits == nullptr) return BSATTN_ERR_NULL;
+  if (Bm <= 0 || Hm <= 0 || nb <= 0 || valid_last < 1 || valid_last > BSATTN_TILE) return BSATTN_ERR_SHAPE;
+  if ((int64_t)Bm * Hm * nb > 0x7fffffff) return BSATTN_ERR_RANGE;
+  return launch_tail_tiles(Bm, Hm, nb, valid_last, transposed != 0, row_ptr, col_idx, tile_partial,
+                           (unsigned long long*)tile_bits, (hipStream_t)stream);
+}
+
 static int check_attn(int Bm, int Hm, int B, int H, int N, int D, int dtype, int out_dtype) {
   if (B <= 0 || H <= 0 || N <= 0 || N % BSATTN_TILE != 0) return BSATTN_ERR_SHAPE;
   if (!((Bm == 1 || Bm == B) && (Hm == 1 || Hm == H))) return BSATTN_ERR_SHAPE;

@@ -15,6 +15,8 @@ int launch_block_mask_to_lists(const uint8_t* block, int Bm, int Hm, int nb, int
                                int64_t sm, int64_t sn, int32_t* row_ptr, int32_t* col_idx,
                                int32_t* groups, int32_t* counts, int32_t* ws, hipStream_t st);
 
+int launch_tail_tiles(int Bm, int Hm, int nb, int valid, int transpose, const int32_t* row_ptr,
+                      const int32_t* col_idx, uint8_t* partial, unsigned long long* bits, hipStream_t st);
 int launch_pack_tiles(const uint8_t* dense, int Bm, int Hm, int nb, int64_t sb, int64_t sh, int64_t sm,
                       int64_t sn, const int32_t* row_ptr, const int32_t* col_idx, uint8_t* partial,
                       unsigned long long* bits, hipStream_t st);

@@ -177,6 +177,35 @@ int launch_block_mask_to_lists(const uint8_t* block, int Bm, int Hm, int nb, int
   return launch_status();
 }
 
+// Sequence lengths that are not a multiple of 64: the last column block holds only `valid` keys.
+// One workgroup per list row (mask head, block a); for each of its kept tiles the flag and the 64
+// words in the format of pack_tiles_kernel: all ones, except in the last column block, where
+// (row lists) every word keeps its low `valid` bits or (column lists: word = key, bit = query)
+// only the first `valid` words are set.
+__global__ __launch_bounds__(256) void tail_tiles_kernel(const int32_t* __restrict__ row_ptr,
+                                                         const int32_t* __restrict__ col_idx, int nb, int valid,
+                                                         int transpose, uint8_t* __restrict__ partial,
+                                                         unsigned long long* __restrict__ bits) {
+  const int r = blockIdx.x, a = r % nb;
+  const int t0 = row_ptr[r], t1 = row_ptr[r + 1];
+  const unsigned long long ones = ~0ull, low = valid >= 64 ? ones : ((1ull << valid) - 1ull);
+  for (int i = threadIdx.x; i < (t1 - t0) * 64; i += 256) {
+    const int t = t0 + (i >> 6), w = i & 63;
+    const bool last = transpose ? a == nb - 1 : col_idx[t] == nb - 1;
+    unsigned long long word = ones;
+    if (last) word = transpose ? (w < valid ? ones : 0ull) : low;
+    bits[(int64_t)t * 64 + w] = word;
+    if (w == 0) partial[t] = last && valid < 64 ? 1 : 0;
+  }
+}
+
+int launch_tail_tiles(int Bm, int Hm, int nb, int valid, int transpose, const int32_t* row_ptr,
+                      const int32_t* col_idx, uint8_t* partial, unsigned long long* bits, hipStream_t st) {
+  hipLaunchKernelGGL(tail_tiles_kernel, dim3(Bm * Hm * nb), dim3(256), 0, st, row_ptr, col_idx, nb, valid, transpose,
+                     partial, bits);
+  return launch_status();
+}
+
 int launch_pack_tiles(const uint8_t* dense, int Bm, int Hm, int nb, int64_t sb, int64_t sh, int64_t sm,
                       int64_t sn, const int32_t* row_ptr, const int32_t* col_idx, uint8_t* partial,
                       unsigned long long* bits, hipStream_t st) {

@@ -9,7 +9,7 @@ import ctypes
 import torch
 
 from . import _ext
-from .utils import TILE, block_mask_to_lists, mask_to_lists, to_block_mask, _check_mask
+from .utils import TILE, block_mask_to_lists, mask_to_lists, num_tiles, is_block_form, _check_mask
 
 
 def build_groups_from_block_mask(mask):
@@ -41,16 +41,29 @@ def _check_qkv(q, k, v, mask):
     if q.dtype not in (torch.float16, torch.bfloat16) or k.dtype != q.dtype or v.dtype != q.dtype:
         raise TypeError("q, k, v must all be float16 or all bfloat16")
     B, H, N, D = q.shape
-    if D not in (64, 128):                                             # :58 and fa2_fwd.py:120
-        raise ValueError("head dimension must be 64 or 128")
-    if N % TILE != 0:
-        raise ValueError("sequence length must be a multiple of 64")
+    if D not in (16, 32, 64, 128):                                     # :58 and fa2_fwd.py:120 (256 is not built)
+        raise ValueError("head dimension must be 16, 32, 64 or 128")
+    if N < 1:
+        raise ValueError("empty sequence")
     if mask is None:
         return B, H, N, D
     _check_mask(mask)
     if mask.shape[0] not in (1, B) or mask.shape[1] not in (1, H):
         raise ValueError("mask batch/head sizes must be 1 or match q")
+    is_block_form(mask, N)                                              # raises on any other shape
     return B, H, N, D
+
+
+def _padded(x, N, D):
+    """The kernels work on whole 64-token tiles and on head dimensions 64 and 128: other shapes
+    are embedded in zeros.  Zero columns change neither q k^T nor the real columns of the
+    output; the keys of zero rows are masked (utils.mask_to_lists), their query rows are dropped."""
+    Np, Dp = num_tiles(N) * TILE, (64 if D < 64 else D)
+    if (Np, Dp) == (x.shape[2], x.shape[3]):
+        return x
+    xp = x.new_zeros((x.shape[0], x.shape[1], Np, Dp))
+    xp[:, :, :x.shape[2], :x.shape[3]] = x
+    return xp
 
 
 _all_true = {}
@@ -91,6 +104,8 @@ class ForwardPlan:
 
     def __init__(self, q, k, v, lists, sm_scale, out_dtype=None, stream=None):
         B, H, N, D = q.shape
+        if N % TILE or D not in (64, 128):
+            raise ValueError("a plan takes whole tiles only: N % 64 == 0 and D in {64, 128}")
         self.q, self.k, self.v, self.lists = _prep(q), _prep(k), _prep(v), lists
         out_dtype = out_dtype or q.dtype
         self.o = torch.empty((B, H, N, D), dtype=out_dtype, device=q.device)
@@ -144,15 +159,19 @@ class _attention(torch.autograd.Function):
     def forward(ctx, q, k, v, mask=None, sm_scale=1.3, out_fp32=False, return_lse=False):
         B, H, N, D = _check_qkv(q, k, v, mask)
         if mask is None:
-            mask = _dense_mask(q.device, N // TILE)
+            mask = _dense_mask(q.device, num_tiles(N))
         lists = mask_to_lists(mask, N)                                       # :48
         out_dtype = torch.float32 if out_fp32 else q.dtype
+        q, k, v = _padded(q, N, D), _padded(k, N, D), _padded(v, N, D)
         o, lse = _forward(q, k, v, lists, sm_scale, out_dtype, True)
         ctx.save_for_backward(q, k, v, o, lse, mask)                         # :89
         ctx.lists = lists
         ctx.sm_scale = sm_scale
         ctx.out_dtype = out_dtype
         ctx.return_lse = return_lse
+        ctx.shape = (N, D)
+        if o.shape[2:] != (N, D):
+            o, lse = o[:, :, :N, :D], lse[:, :, :N]
         if return_lse:
             ctx.mark_non_differentiable(lse)
             return o, lse
@@ -161,19 +180,25 @@ class _attention(torch.autograd.Function):
     @staticmethod
     def backward(ctx, do, *unused):
         q, k, v, o, lse, mask = ctx.saved_tensors
-        lists_t = mask_to_lists(mask, q.shape[2], transpose=True)
+        N, D = ctx.shape
+        lists_t = mask_to_lists(mask, N, transpose=True)
         o_in = o if o.dtype == q.dtype else o.to(q.dtype)
-        do_in = do if do.dtype == q.dtype else do.to(q.dtype)
+        do_in = _padded(do if do.dtype == q.dtype else do.to(q.dtype), N, D)
         # autograd hands gradients back in the dtype of q, k, v
         dq, dk, dv = _backward(q, k, v, o_in, do_in, lse, ctx.lists, lists_t, ctx.sm_scale, q.dtype)
+        if dq.shape[2:] != (N, D):
+            dq, dk, dv = dq[:, :, :N, :D], dk[:, :, :N, :D], dv[:, :, :N, :D]
         return dq, dk, dv, None, None, None, None                            # :155
 
 
 def flash_attention_custom_mask(q, k, v, mask=None, sm_scale=1.3):
     """Drop-in for the reference's `flash_attention_custom_mask = _attention.apply`
     (fa2_custom_mask.py:157): q,k,v [B,H,N,D] fp16/bf16 on the GPU, mask bool
-    [B|1,H|1,N/64,N/64] (or elementwise [B|1,H|1,N,N]; None = dense attention), returns o like
-    q.  The kept-tile lists of a mask tensor are cached until the tensor is modified."""
+    [B|1,H|1,nb,nb] with nb = ceil(N/64) (or elementwise [B|1,H|1,N,N]; None = dense attention),
+    returns o like q.  D is 16, 32, 64 or 128; N need not be a multiple of 64 (the last block of a
+    block mask then covers the remaining tokens).  Shapes other than D in {64,128}, N % 64 == 0
+    cost one zero-padded copy of q, k, v per call.  The kept-tile lists of a mask tensor are cached
+    until the tensor is modified."""
     return _attention.apply(q, k, v, mask, sm_scale)
 
 
@@ -189,11 +214,15 @@ def attention_forward_backward(q, k, v, mask, sm_scale, do, out_fp32=False):
     are fp32 (autograd itself can only hand back gradients in the dtype of q)."""
     B, H, N, D = _check_qkv(q, k, v, mask)
     if mask is None:
-        mask = _dense_mask(q.device, N // TILE)
+        mask = _dense_mask(q.device, num_tiles(N))
     lists = mask_to_lists(mask, N)
     lists_t = mask_to_lists(mask, N, transpose=True)
     out_dtype = torch.float32 if out_fp32 else q.dtype
+    q, k, v = _padded(q, N, D), _padded(k, N, D), _padded(v, N, D)
     o, lse = _forward(q, k, v, lists, sm_scale, out_dtype, True)
     o_in = o if o.dtype == q.dtype else o.to(q.dtype)
-    dq, dk, dv = _backward(q, k, v, o_in, do.to(q.dtype), lse, lists, lists_t, sm_scale, out_dtype)
+    dq, dk, dv = _backward(q, k, v, o_in, _padded(do.to(q.dtype), N, D), lse, lists, lists_t, sm_scale, out_dtype)
+    if o.shape[2:] != (N, D):
+        o, lse = o[:, :, :N, :D], lse[:, :, :N]
+        dq, dk, dv = dq[:, :, :N, :D], dk[:, :, :N, :D], dv[:, :, :N, :D]
     return o, lse, dq, dk, dv

@@ -116,16 +116,42 @@ def pack_mask_tiles(mask, lists, transpose=False):
     return partial, bits
 
 
-def to_block_mask(mask, N):
-    """Accepts the reference's block form [.,.,N/64,N/64] or an elementwise [.,.,N,N] mask."""
-    _check_mask(mask)
-    nb = N // TILE
-    if mask.shape[2] == nb and mask.shape[3] == nb:
-        return mask
+def tail_mask_tiles(lists, valid_last, transpose=False):
+    """Words of the kept tiles of a block mask whose last column block holds only `valid_last`
+    real keys (sequence length not a multiple of 64): (tile_partial, tile_bits) in the format of
+    pack_mask_tiles, every tile completely set except for the padding keys."""
+    dev = lists.row_ptr.device
+    cap = lists.Bm * lists.Hm * lists.nb * lists.nb
+    partial = torch.empty(cap, dtype=torch.uint8, device=dev)
+    bits = torch.empty((cap, 64), dtype=torch.int64, device=dev)
+    rc = _ext.lib().bsattn_tail_mask_tiles(lists.Bm, lists.Hm, lists.nb, valid_last, 1 if transpose else 0,
+                                           lists.row_ptr.data_ptr(), lists.col_idx.data_ptr(), partial.data_ptr(),
+                                           bits.data_ptr(), _ext.current_stream(dev))
+    _ext.check(rc, "bsattn_tail_mask_tiles")
+    return partial, bits
+
+
+def num_tiles(N):
+    """Row (and column) blocks of a sequence of N tokens; the last one may be partly filled."""
+    return -(-N // TILE)
+
+
+def is_block_form(mask, N):
+    """True for the reference's block form [.,.,nb,nb], False for an elementwise [.,.,N,N] mask."""
+    nb = num_tiles(N)
+    if mask.shape[2] == nb and mask.shape[3] == nb and N != nb:
+        return True
     if mask.shape[2] == N and mask.shape[3] == N:
-        return reduce_dense_mask(mask)
+        return False
     raise ValueError("mask shape %s matches neither [.., %d, %d] nor [.., %d, %d]"
                      % (tuple(mask.shape), nb, nb, N, N))
+
+
+def to_block_mask(mask, N):
+    """Accepts the reference's block form [.,.,N/64,N/64] or an elementwise [.,.,N,N] mask
+    (N a multiple of 64)."""
+    _check_mask(mask)
+    return mask if is_block_form(mask, N) else reduce_dense_mask(mask)
 
 
 class _ListsCache:
@@ -161,8 +187,15 @@ def mask_to_lists(mask, N, transpose=False):
     """TileLists of a block or elementwise mask for sequence length N, through the cache."""
     lists = lists_cache.get(mask, N, transpose)
     if lists is None:
-        lists = block_mask_to_lists(to_block_mask(mask, N), transpose=transpose)
-        if mask.shape[2] == N and N != N // TILE:          # elementwise form: exact inside tiles
-            lists.partial, lists.bits = pack_mask_tiles(mask, lists, transpose=transpose)
+        _check_mask(mask)
+        pad = num_tiles(N) * TILE - N          # > 0: q, k, v get `pad` zero rows, whose keys are masked here
+        if is_block_form(mask, N):
+            lists = block_mask_to_lists(mask, transpose=transpose)
+            if pad:
+                lists.partial, lists.bits = tail_mask_tiles(lists, TILE - pad, transpose=transpose)
+        else:                                  # elementwise form: exact inside tiles
+            dense = torch.nn.functional.pad(mask, (0, pad, 0, pad)) if pad else mask
+            lists = block_mask_to_lists(reduce_dense_mask(dense), transpose=transpose)
+            lists.partial, lists.bits = pack_mask_tiles(dense, lists, transpose=transpose)
         lists_cache.put(mask, N, transpose, lists)
     return lists

@@ -99,6 +99,18 @@ int bsattn_pack_mask_tiles(const uint8_t* dense, int Bm, int Hm, int N, int64_t 
                            int64_t sm, int64_t sn, const int32_t* row_ptr, const int32_t* col_idx,
                            uint8_t* tile_partial, uint64_t* tile_bits, void* stream);
 
+/* Sequence lengths N that are not a multiple of 64 (unsupported by the reference, whose block
+ * pointers assume whole tiles: fa2_custom_mask/fa2_fwd.py:137-172): the caller pads q, k, v
+ * with zero rows to nb*64 tokens and masks the padding keys through the elementwise entry
+ * points.  This fills tile_partial / tile_bits (same format and capacity as
+ * bsattn_pack_mask_tiles) for the lists of a block mask [Bm,Hm,nb,nb] whose last column block
+ * holds only valid_last (1..64) real keys: every tile is completely set except those of the
+ * last column block, which keep their first valid_last keys.  transposed != 0: row_ptr /
+ * col_idx are the column lists (the words the dK/dV pass uses). */
+int bsattn_tail_mask_tiles(int Bm, int Hm, int nb, int valid_last, int transposed,
+                           const int32_t* row_ptr, const int32_t* col_idx, uint8_t* tile_partial,
+                           uint64_t* tile_bits, void* stream);
+
 /* ------------------------------------------------------------------------------------
  * Forward.  Replaces the launch of _attn_fwd (fa2_custom_mask/fa2_fwd.py:108-206) from
  * _attention.forward (fa2_custom_mask/fa2_custom_mask.py:69-87).

@@ -63,6 +63,9 @@ def test_argument_validation_without_gpu():
     assert l.bsattn_reduce_dense_mask(P, 1, 1, 64, 0, 0, 72, P, None) == -5
     assert l.bsattn_block_mask_to_lists(P, 1, 1, 4, 16, 16, 4, 1, P, P, None, P, None, 0, None) == -6
     assert l.bsattn_block_mask_to_lists(P, 1, 1, 4, 16, 16, 4, 1, None, P, None, P, P, 64, None) == -1
+    assert l.bsattn_tail_mask_tiles(1, 1, 4, 0, 0, P, P, P, P, None) == -2       # 1..64 valid keys
+    assert l.bsattn_tail_mask_tiles(1, 1, 4, 65, 0, P, P, P, P, None) == -2
+    assert l.bsattn_tail_mask_tiles(1, 1, 4, 10, 0, P, None, P, P, None) == -1
     assert l.bsattn_reorder(P, P, 1, 1, 2, 2, 2, 3, 2, P, None, None) == -5      # 6-byte rows
     assert l.bsattn_reorder(P, P, 1, 1, 0, 2, 2, 4, 2, P, None, None) == -2
     assert l.bsattn_reorder(P, P, 1, 1, 2, 2, 2, 4, 2, None, None, None) == -1
