@@ -103,3 +103,24 @@ def test_mfma_rate_probe_runs(dev):
     assert flops.value == cus * 8 * 4 * 8 * 2 * 32 * 32 * 16
     # every accumulator element is 4 iterations x 2 MFMAs per chain x 16 ones = 128; 64 elements per lane
     assert torch.all(sink == 128.0 * 64)
+
+
+def test_committed_toy_fixture(dev):
+    """Forward, LSE and gradients against tests/golden/toy_attention_fixture.npz (float64 torch on the CPU):
+    both heads through the elementwise mask, head 0 also through the block form of its mask."""
+    import os
+    import fa2_custom_mask as fm
+    fx = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "toy_attention_fixture.npz"))
+    q, k, v, do = [torch.from_numpy(fx[n]).to(dev) for n in ("q", "k", "v", "do")]
+    sc = float(fx["sm_scale"])
+    mask = torch.from_numpy(fx["mask"]).to(dev)
+    res = fm.attention_forward_backward(q, k, v, mask, sc, do, out_fp32=True)
+    for got, name in zip(res, ("o", "lse", "dq", "dk", "dv")):
+        ma, rl = errors(got, fx[name])
+        print("%s max-abs %.3e rel-L2 %.3e" % (name, ma, rl))
+        assert ma <= 2e-2 and rl <= 1e-3, name
+    bm = torch.from_numpy(fx["block_mask_head0"]).reshape(1, 1, 2, 2).to(dev)
+    res0 = fm.attention_forward_backward(q[:, :1], k[:, :1], v[:, :1], bm, sc, do[:, :1], out_fp32=True)
+    for got, name in zip(res0, ("o", "lse", "dq", "dk", "dv")):
+        ma, rl = errors(got, fx[name][:, :1])
+        assert ma <= 2e-2 and rl <= 1e-3, name

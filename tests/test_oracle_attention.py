@@ -176,3 +176,27 @@ def test_elementwise_rows_without_keys_give_zero():
     m[0, 0, 5, :] = False
     o, lse = orc.naive_attention(q, k, v, m, 0.5, return_lse=True)
     assert np.all(o[0, 0, 5] == 0) and lse[0, 0, 5] == -np.inf and np.isfinite(lse[0, 0, 4])
+
+
+def test_oracle_matches_committed_toy_fixture():
+    """tests/golden/toy_attention_fixture.npz holds O, LSE and gradients of a seeded toy problem computed in
+    float64 by torch (naive formula of kernel-test.py:37-40 + autograd), one head with a block mask and one
+    with an elementwise mask."""
+    import os
+    fx = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "toy_attention_fixture.npz"))
+    q, k, v, do = [fx[n].astype(np.float32) for n in ("q", "k", "v", "do")]
+    sc = float(fx["sm_scale"])
+    o, lse = orc.naive_attention(q, k, v, fx["mask"], sc, return_lse=True)
+    assert np.abs(o - fx["o"]).max() <= 2e-6 and np.abs(lse - fx["lse"]).max() <= 2e-6
+    for got, name in zip(orc.attention_backward(q, k, v, fx["mask"], sc, do), ("dq", "dk", "dv")):
+        assert np.abs(got - fx[name]).max() <= 2e-5, name
+    # head 0 through the block form of its mask, numpy and C restatements
+    bm = fx["block_mask_head0"].reshape(1, 1, 2, 2)
+    o0 = orc.naive_attention(q[:, :1], k[:, :1], v[:, :1], bm, sc)
+    assert np.abs(o0 - fx["o"][:, :1]).max() <= 2e-6
+    oc, lc = c_oracle.naive_fwd(q[:, :1], k[:, :1], v[:, :1], bm, sc, 0, 128)
+    assert np.abs(oc - fx["o"][:, :1]).max() <= 2e-6 and np.abs(lc - fx["lse"][:, :1]).max() <= 2e-6
+    groups, n_list = orc.build_groups_from_block_mask(bm)
+    ot = orc.tiled_attention(q[:, :1], k[:, :1], v[:, :1], groups, n_list, sc)
+    ot = ot[0] if isinstance(ot, tuple) else ot
+    assert np.abs(ot - fx["o"][:, :1]).max() <= 2e-6
