@@ -256,7 +256,7 @@ def main():
         "elementwise_mask": elementwise_case(torch, dev, fm, qd, kd, vd, sm_scale),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "fwd_kernel<64,false,false> (one bsattn_fwd call)",
+                     "kernel": "fwd_kernel<64, 0, false, false> (fp16, one bsattn_fwd call)",
                      "algorithmic_flops_per_launch": tile_flops(kept[1.0])},
     }
     if not args.no_cpu:

@@ -128,15 +128,6 @@ __device__ __forceinline__ uintx4 frag_cols(const unsigned char* tile, int db, i
   return a;
 }
 
-__device__ __forceinline__ floatx16 mfma_f16(uintx4 a, uintx4 b, floatx16 c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), c, 0, 0, 0);
-}
-
-__device__ __forceinline__ unsigned int pack_half2(float a, float b) {
-  const half2v h = {(_Float16)a, (_Float16)b};
-  return __builtin_bit_cast(unsigned int, h);
-}
-
 // scores of unset mask elements become -inf; mw: the 64 mask bits of this lane's row, already
 // shifted right by 4 g, so that bit 8(i/4) + i%4 (+ 32 for the second block) belongs to register i
 __device__ __forceinline__ void mask_scores(floatx16& s0, floatx16& s1, unsigned long long mw) {
@@ -171,7 +162,9 @@ __device__ __forceinline__ void head_and_block(int L, int BH, int nb, int& bh, i
 // ---------------------------------------------------------------------------------------
 // dQ: workgroup = row block m, wavefront wv owns queries 64m + 32wv + ln
 // ---------------------------------------------------------------------------------------
-template <int D, bool BF16, bool EW>
+// PB (bf16 inputs only): dS is rounded to bf16 and the second product runs in bf16 on the tile as it
+// is; otherwise dS is rounded to fp16 and bf16 tiles are converted fragment by fragment.
+template <int D, bool BF16, bool EW, bool PB>
 __global__ __launch_bounds__(128) void dq_kernel(const BwdParams prm) {
   using C = BwdCfg<D, EW>;
   constexpr int KS = D / 16, DB = D / 32;
@@ -264,7 +257,7 @@ __global__ __launch_bounds__(128) void dq_kernel(const BwdParams prm) {
 #pragma unroll
     for (int ts = 0; ts < 4; ++ts)
 #pragma unroll
-      for (int db = 0; db < DB; ++db) fkt[ts][db] = frag_cols<D, BF16>(kt, db, ts, lane);
+      for (int db = 0; db < DB; ++db) fkt[ts][db] = frag_cols<D, BF16 && !PB>(kt, db, ts, lane);
     __builtin_amdgcn_sched_barrier(0);
     // dS^T = P^T * (dP^T - delta), this lane's query; packed as operand slices of 16 keys
     uintx4 dsf[4];
@@ -275,13 +268,13 @@ __global__ __launch_bounds__(128) void dq_kernel(const BwdParams prm) {
         const int kb = ts >> 1, i = 8 * (ts & 1) + 2 * jj;
         const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][i], qk_scale, -lse2));
         const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][i + 1], qk_scale, -lse2));
-        dsf[ts][jj] = pack_half2(p0 * (dpacc[kb][i] - dlt), p1 * (dpacc[kb][i + 1] - dlt));
+        dsf[ts][jj] = pack2<PB>(p0 * (dpacc[kb][i] - dlt), p1 * (dpacc[kb][i + 1] - dlt));
       }
 #pragma unroll
     for (int ts = 0; ts < 4; ++ts)
 #pragma unroll
       for (int db = 0; db < DB; ++db)
-        dqacc[db] = mfma_f16(fkt[ts][db], dsf[ts], dqacc[db]);          // dQ^T += K^T dS^T
+        dqacc[db] = mfma_qk<PB>(fkt[ts][db], dsf[ts], dqacc[db]);       // dQ^T += K^T dS^T
   }
 
   void* base = prm.out_f32 ? (void*)((float*)prm.dq + (int64_t)bh * prm.N * D) : (void*)((unsigned short*)prm.dq + (int64_t)bh * prm.N * D);
@@ -297,7 +290,7 @@ __global__ __launch_bounds__(128) void dq_kernel(const BwdParams prm) {
 // ---------------------------------------------------------------------------------------
 // dK, dV: workgroup = column block n, wavefront wv owns keys 64n + 32wv + ln
 // ---------------------------------------------------------------------------------------
-template <int D, bool BF16, bool EW>
+template <int D, bool BF16, bool EW, bool PB>
 __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
   using C = BwdCfg<D, EW>;
   constexpr int KS = D / 16, DB = D / 32;
@@ -389,8 +382,8 @@ __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
     for (int ts = 0; ts < 4; ++ts)
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        fgt[ts][db] = frag_cols<D, BF16>(gt, db, ts, lane);
-        fqt[ts][db] = frag_cols<D, BF16>(qt, db, ts, lane);
+        fgt[ts][db] = frag_cols<D, BF16 && !PB>(gt, db, ts, lane);
+        fqt[ts][db] = frag_cols<D, BF16 && !PB>(qt, db, ts, lane);
       }
     __builtin_amdgcn_sched_barrier(0);
     // rows of the results are queries: register i of block qb <-> query 32qb + 8(i/4) + 4g + i%4
@@ -411,15 +404,15 @@ __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
           p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[qb][i0 + e], qk_scale, nl));
           ds[e] = p[e] * (dpacc[qb][i0 + e] - d4[e]);
         }
-        pf[ts][2 * jh] = pack_half2(p[0], p[1]);   pf[ts][2 * jh + 1] = pack_half2(p[2], p[3]);
-        dsf[ts][2 * jh] = pack_half2(ds[0], ds[1]); dsf[ts][2 * jh + 1] = pack_half2(ds[2], ds[3]);
+        pf[ts][2 * jh] = pack2<PB>(p[0], p[1]);   pf[ts][2 * jh + 1] = pack2<PB>(p[2], p[3]);
+        dsf[ts][2 * jh] = pack2<PB>(ds[0], ds[1]); dsf[ts][2 * jh + 1] = pack2<PB>(ds[2], ds[3]);
       }
 #pragma unroll
     for (int ts = 0; ts < 4; ++ts)
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        dvacc[db] = mfma_f16(fgt[ts][db], pf[ts], dvacc[db]);    // dV^T += dO^T P
-        dkacc[db] = mfma_f16(fqt[ts][db], dsf[ts], dkacc[db]);   // dK^T += Q^T dS
+        dvacc[db] = mfma_qk<PB>(fgt[ts][db], pf[ts], dvacc[db]);    // dV^T += dO^T P
+        dkacc[db] = mfma_qk<PB>(fqt[ts][db], dsf[ts], dkacc[db]);   // dK^T += Q^T dS
       }
   }
 
@@ -446,14 +439,14 @@ size_t bwd_workspace_bytes(int B, int H, int N, int D) {
   return (size_t)B * H * N * sizeof(float);   // delta
 }
 
-template <int D, bool BF16, bool EW>
+template <int D, bool BF16, bool EW, bool PB>
 static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
   using C = BwdCfg<D, EW>;
   static bool configured = false;   // raising the dynamic LDS limit is idempotent
   if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dq_kernel<D, BF16, EW>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dq_kernel<D, BF16, EW, PB>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv_kernel<D, BF16, EW>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv_kernel<D, BF16, EW, PB>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
     configured = true;
   }
@@ -461,8 +454,8 @@ static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
   constexpr int RPB = 256 / (D / 8);
   hipLaunchKernelGGL((delta_kernel<D, BF16>), dim3((prm.N + RPB - 1) / RPB, BH), dim3(256), 0, st, prm);
   const int grid = ((BH + 7) / 8) * 8 * prm.nb;   // heads in groups of 8, the last group padded
-  hipLaunchKernelGGL((dq_kernel<D, BF16, EW>), dim3(grid), dim3(128), C::LDS_BYTES, st, prm);
-  hipLaunchKernelGGL((dkdv_kernel<D, BF16, EW>), dim3(grid), dim3(128), C::LDS_BYTES, st, prm);
+  hipLaunchKernelGGL((dq_kernel<D, BF16, EW, PB>), dim3(grid), dim3(128), C::LDS_BYTES, st, prm);
+  hipLaunchKernelGGL((dkdv_kernel<D, BF16, EW, PB>), dim3(grid), dim3(128), C::LDS_BYTES, st, prm);
 }
 
 int launch_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
@@ -483,16 +476,24 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* o, const
     prm.qs[i] = s.qs[i]; prm.ks[i] = s.ks[i]; prm.vs[i] = s.vs[i]; prm.os[i] = s.os[i]; prm.dos[i] = s.dos[i];
   }
   const bool bf = s.dtype == BSATTN_BF16;
+  // bf16 gradients are rounded to 8 bits anyway: P and dS are then rounded to bf16 as well (what the
+  // reference's forward does with P, fa2_fwd.py:189) and no tile needs converting; fp32 gradients of
+  // bf16 inputs keep P and dS in fp16.
+  const bool pb = bf && !prm.out_f32;
   if (bits_rows == nullptr) {
-    if (s.D == 64 && !bf) launch_bwd_t<64, false, false>(prm, st);
-    else if (s.D == 64 && bf) launch_bwd_t<64, true, false>(prm, st);
-    else if (s.D == 128 && !bf) launch_bwd_t<128, false, false>(prm, st);
-    else launch_bwd_t<128, true, false>(prm, st);
+    if (s.D == 64 && !bf) launch_bwd_t<64, false, false, false>(prm, st);
+    else if (s.D == 64 && pb) launch_bwd_t<64, true, false, true>(prm, st);
+    else if (s.D == 64) launch_bwd_t<64, true, false, false>(prm, st);
+    else if (s.D == 128 && !bf) launch_bwd_t<128, false, false, false>(prm, st);
+    else if (pb) launch_bwd_t<128, true, false, true>(prm, st);
+    else launch_bwd_t<128, true, false, false>(prm, st);
   } else {   // elementwise mask
-    if (s.D == 64 && !bf) launch_bwd_t<64, false, true>(prm, st);
-    else if (s.D == 64 && bf) launch_bwd_t<64, true, true>(prm, st);
-    else if (s.D == 128 && !bf) launch_bwd_t<128, false, true>(prm, st);
-    else launch_bwd_t<128, true, true>(prm, st);
+    if (s.D == 64 && !bf) launch_bwd_t<64, false, true, false>(prm, st);
+    else if (s.D == 64 && pb) launch_bwd_t<64, true, true, true>(prm, st);
+    else if (s.D == 64) launch_bwd_t<64, true, true, false>(prm, st);
+    else if (s.D == 128 && !bf) launch_bwd_t<128, false, true, false>(prm, st);
+    else if (pb) launch_bwd_t<128, true, true, true>(prm, st);
+    else launch_bwd_t<128, true, true, false>(prm, st);
   }
   return launch_status();
 }

@@ -59,9 +59,11 @@ template <int D> struct FwdCfg {
   static constexpr int SHORT_ROW = 6 * NW;                  // row blocks up to this many tiles may go to one wavefront
 };
 
-template <int D, bool BF16, bool ROWS, bool EW>
+// DT: 0 fp16; 1 bf16 with P rounded to fp16 (V fragments converted); 2 bf16 with P rounded to bf16.
+template <int D, int DT, bool ROWS, bool EW>
 __global__ __launch_bounds__(FwdCfg<D>::NW * 64, FwdCfg<D>::WG_PER_CU)
 void fwd_kernel(const FwdParams prm) {
+  constexpr bool BF16 = DT != 0, PB = DT == 2;
   using C = FwdCfg<D>;
   constexpr int NW = C::NW;
   constexpr bool FOLD = !BF16;     // fp16: scale folded into Q, reference exponent via an extra MFMA slice
@@ -261,7 +263,7 @@ void fwd_kernel(const FwdParams prm) {
             const uintx2 r2 = __builtin_bit_cast(uintx2, rr);
             a[2 * jh] = r2[0]; a[2 * jh + 1] = r2[1];
           }
-          if constexpr (BF16) a = bf16x8_to_f16x8(a);
+          if constexpr (BF16 && !PB) a = bf16x8_to_f16x8(a);
           vfr[ts][db] = a;
         }
     };
@@ -270,9 +272,7 @@ void fwd_kernel(const FwdParams prm) {
       for (int ts = 0; ts < 4; ++ts)
 #pragma unroll
         for (int db = 0; db < DB; ++db)
-          oacc[db][qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, vfr[ts][db]),
-                                                               __builtin_bit_cast(half8, pf[ts][qb]),
-                                                               oacc[db][qb], 0, 0, 0);
+          oacc[db][qb] = mfma_qk<PB>(vfr[ts][db], pf[ts][qb], oacc[db][qb]);
     };
     // Softmax numerators, one query per lane.  Fast path: P = exp2(score - m_i) with the
     // reference m_i left alone; the row sum of the fp16-rounded P (what the second product
@@ -282,7 +282,7 @@ void fwd_kernel(const FwdParams prm) {
     auto settle = [&](int qb, floatx16& s0, floatx16& s1, float lnew) {
       if (__any(fresh || (EW && l_i[qb] == 0.f) || !(lnew - l_i[qb] < 16384.0f))) {
         recentre<DB, FOLD, EW>(s0, s1, oacc, qb, qk_scale, m_i[qb], l_i[qb], mfrag[qb], fresh, g);
-        lnew = softmax_tile<FOLD>(s0, s1, qk_scale, m_i[qb], l_i[qb], pf, qb);
+        lnew = softmax_tile<FOLD, PB>(s0, s1, qk_scale, m_i[qb], l_i[qb], pf, qb);
       }
       l_i[qb] = lnew;
     };
@@ -318,7 +318,7 @@ void fwd_kernel(const FwdParams prm) {
     // [2]
     scores(1, sb0, sb1);
     if constexpr (EW) { if (partial) mask_scores(sb0, sb1, mw1); }
-    float lnew0 = softmax_tile<FOLD>(sa0, sa1, qk_scale, m_i[0], l_i[0], pf, 0);
+    float lnew0 = softmax_tile<FOLD, PB>(sa0, sa1, qk_scale, m_i[0], l_i[0], pf, 0);
 #pragma unroll
     for (int it = 0; it < 2 * KS + (FOLD ? 2 : 0); ++it) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
@@ -332,7 +332,7 @@ void fwd_kernel(const FwdParams prm) {
     if (copy_v) v_copy_all(vg + (int64_t)cbn * 64 * prm.vs[2]);
     // [3]
     second(0);
-    float lnew1 = softmax_tile<FOLD>(sb0, sb1, qk_scale, m_i[1], l_i[1], pf, 1);
+    float lnew1 = softmax_tile<FOLD, PB>(sb0, sb1, qk_scale, m_i[1], l_i[1], pf, 1);
 #pragma unroll
     for (int it = 0; it < 4 * DB; ++it) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -814,21 +814,21 @@ static bool use_pair_kernel(int64_t row_blocks, int nb) {
 // wavefront takes whole row blocks, which needs no merge and no second kernel.
 static bool rows_mode(const FwdParams& prm) { return prm.nb >= 8 * prm.W; }
 
-template <int D, bool BF16, bool EW>
+template <int D, int DT, bool EW>
 static void launch_fwd_t(const FwdParams& prm, int BH, hipStream_t st) {
   using C = FwdCfg<D>;
   static bool configured = false;   // raising the dynamic LDS limit is idempotent
   if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<D, BF16, false, EW>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<D, DT, false, EW>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<D, BF16, true, EW>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<D, DT, true, EW>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
     configured = true;
   }
   if (rows_mode(prm)) {
-    hipLaunchKernelGGL((fwd_kernel<D, BF16, true, EW>), dim3(prm.W * BH), dim3(C::NW * 64), C::LDS_BYTES, st, prm);
+    hipLaunchKernelGGL((fwd_kernel<D, DT, true, EW>), dim3(prm.W * BH), dim3(C::NW * 64), C::LDS_BYTES, st, prm);
   } else {
-    hipLaunchKernelGGL((fwd_kernel<D, BF16, false, EW>), dim3(prm.W * BH), dim3(C::NW * 64), C::LDS_BYTES, st, prm);
+    hipLaunchKernelGGL((fwd_kernel<D, DT, false, EW>), dim3(prm.W * BH), dim3(C::NW * 64), C::LDS_BYTES, st, prm);
   }
 }
 
@@ -851,19 +851,18 @@ int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
   const bool bf = s.dtype == BSATTN_BF16;
   const int BH = s.B * s.H;
   if (s.D == 128 && use_pair_kernel((int64_t)BH * prm.nb, prm.nb)) {
-    launch_fwd_pair(prm, bf ? 1 : 0, tile_bits != nullptr, st);
+    launch_fwd_pair(prm, !bf ? 0 : (prm.out_f32 ? 1 : 2), tile_bits != nullptr, st);
     return launch_status();
   }
+  // bf16 with a bf16-typed result: P is rounded to bf16 as well (the reference rounds P to the type of
+  // V, fa2_fwd.py:189) and V is used as it is; an fp32 result keeps P in fp16
+  const int dt = !bf ? 0 : (prm.out_f32 ? 1 : 2);
   if (tile_bits == nullptr) {
-    if (s.D == 64 && !bf) launch_fwd_t<64, false, false>(prm, BH, st);
-    else if (s.D == 64 && bf) launch_fwd_t<64, true, false>(prm, BH, st);
-    else if (s.D == 128 && !bf) launch_fwd_t<128, false, false>(prm, BH, st);
-    else launch_fwd_t<128, true, false>(prm, BH, st);
-  } else {   // elementwise mask: kernels that apply the packed mask words inside partly set tiles
-    if (s.D == 64 && !bf) launch_fwd_t<64, false, true>(prm, BH, st);
-    else if (s.D == 64 && bf) launch_fwd_t<64, true, true>(prm, BH, st);
-    else if (s.D == 128 && !bf) launch_fwd_t<128, false, true>(prm, BH, st);
-    else launch_fwd_t<128, true, true>(prm, BH, st);
+    if (s.D == 64) { if (dt == 0) launch_fwd_t<64, 0, false>(prm, BH, st); else if (dt == 1) launch_fwd_t<64, 1, false>(prm, BH, st); else launch_fwd_t<64, 2, false>(prm, BH, st); }
+    else { if (dt == 0) launch_fwd_t<128, 0, false>(prm, BH, st); else if (dt == 1) launch_fwd_t<128, 1, false>(prm, BH, st); else launch_fwd_t<128, 2, false>(prm, BH, st); }
+  } else {   // elementwise mask
+    if (s.D == 64) { if (dt == 0) launch_fwd_t<64, 0, true>(prm, BH, st); else if (dt == 1) launch_fwd_t<64, 1, true>(prm, BH, st); else launch_fwd_t<64, 2, true>(prm, BH, st); }
+    else { if (dt == 0) launch_fwd_t<128, 0, true>(prm, BH, st); else if (dt == 1) launch_fwd_t<128, 1, true>(prm, BH, st); else launch_fwd_t<128, 2, true>(prm, BH, st); }
   }
   return launch_status();
 }

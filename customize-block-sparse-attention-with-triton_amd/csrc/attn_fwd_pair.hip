@@ -25,6 +25,7 @@ template <int DT, bool EW>
 __global__ __launch_bounds__(128, 2) void fwd_pair_kernel(const FwdParams prm) {
   constexpr int D = 128, KS = D / 16, DB = D / 32, CPR = D / 8, ROWB = 2 * D, TILE_BYTES = 64 * ROWB;
   constexpr bool BF16 = DT != 0;
+  constexpr bool PB = DT == 2;                   // P rounded to bf16, second product in bf16 (V as it is)
   constexpr bool FOLD = !BF16;
   constexpr int HALF = CPR / 2;                  // copy instructions per wavefront and tile
   constexpr int KOPS = HALF + (EW ? 1 : 0), VOPS = HALF;
@@ -207,10 +208,10 @@ __global__ __launch_bounds__(128, 2) void fwd_pair_kernel(const FwdParams prm) {
     }
     // ---- softmax numerators ----
     uintx4 pf[4][2];
-    float lnew = softmax_tile<FOLD>(s0, s1, qk_scale, m_i, l_i, pf, 0);
+    float lnew = softmax_tile<FOLD, PB>(s0, s1, qk_scale, m_i, l_i, pf, 0);
     if (__any(fresh || (EW && l_i == 0.f) || !(lnew - l_i < 16384.0f))) {
       recentre<DB, FOLD, EW>(s0, s1, oacc, 0, qk_scale, m_i, l_i, mfrag, fresh, g);
-      lnew = softmax_tile<FOLD>(s0, s1, qk_scale, m_i, l_i, pf, 0);
+      lnew = softmax_tile<FOLD, PB>(s0, s1, qk_scale, m_i, l_i, pf, 0);
     }
     l_i = lnew;
     fresh = false;
@@ -232,7 +233,7 @@ __global__ __launch_bounds__(128, 2) void fwd_pair_kernel(const FwdParams prm) {
           const uintx2 r2 = __builtin_bit_cast(uintx2, rr);
           a[2 * jh] = r2[0]; a[2 * jh + 1] = r2[1];
         }
-        if constexpr (BF16) a = bf16x8_to_f16x8(a);
+        if constexpr (BF16 && !PB) a = bf16x8_to_f16x8(a);
         vfr[ts][db] = a;
       }
     lds_wait();
@@ -243,8 +244,7 @@ __global__ __launch_bounds__(128, 2) void fwd_pair_kernel(const FwdParams prm) {
     for (int ts = 0; ts < 4; ++ts)
 #pragma unroll
       for (int db = 0; db < DB; ++db)
-        oacc[db][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, vfr[ts][db]),
-                                                            __builtin_bit_cast(half8, pf[ts][0]), oacc[db][0], 0, 0, 0);
+        oacc[db][0] = mfma_qk<PB>(vfr[ts][db], pf[ts][0], oacc[db][0]);
     if (has1) {
       wait_vm<VOPS>();                              // this wavefront's half of K(t+1) has landed (V(t+1) may be in flight)
       __syncthreads();                              // ... and the other half
@@ -279,10 +279,17 @@ static void launch_pair_t(const FwdParams& prm, hipStream_t st) {
   hipLaunchKernelGGL((fwd_pair_kernel<DT, EW>), dim3(grid), dim3(128), PAIR_LDS_BYTES, st, prm);
 }
 
-// D = 128 only.  dt: 0 fp16, 1 bf16.
+// D = 128 only.  dt: 0 fp16, 1 bf16 with P rounded to fp16 (V converted), 2 bf16 with P rounded to bf16.
 void launch_fwd_pair(const FwdParams& prm, int dt, bool elementwise, hipStream_t st) {
-  if (!elementwise) { if (dt == 0) launch_pair_t<0, false>(prm, st); else launch_pair_t<1, false>(prm, st); }
-  else { if (dt == 0) launch_pair_t<0, true>(prm, st); else launch_pair_t<1, true>(prm, st); }
+  if (!elementwise) {
+    if (dt == 0) launch_pair_t<0, false>(prm, st);
+    else if (dt == 1) launch_pair_t<1, false>(prm, st);
+    else launch_pair_t<2, false>(prm, st);
+  } else {
+    if (dt == 0) launch_pair_t<0, true>(prm, st);
+    else if (dt == 1) launch_pair_t<1, true>(prm, st);
+    else launch_pair_t<2, true>(prm, st);
+  }
 }
 
 }  // namespace bsattn

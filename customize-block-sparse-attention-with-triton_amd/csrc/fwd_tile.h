@@ -24,11 +24,10 @@ struct FwdParams {
 // P = exp2(score - m) for the 2 x 16 scores one lane holds of one query (key blocks s0, s1),
 // rounded to fp16 and packed as the operand fragments pf[0..3][qb] of the second product.
 // Returns l + the row sum of the rounded P over this lane's keys.  With FOLD the scores
-// already are "scaled score - m".
-template <bool FOLD>
+// already are "scaled score - m".  PB: P is rounded to bf16 instead of fp16.
+template <bool FOLD, bool PB = false>
 __device__ __forceinline__ float softmax_tile(const floatx16& s0, const floatx16& s1, float qk_scale, float m,
                                               float l, uintx4 (&pf)[4][2], int qb) {
-  const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
 #pragma unroll
   for (int ts = 0; ts < 4; ++ts) {
 #pragma unroll
@@ -37,9 +36,9 @@ __device__ __forceinline__ float softmax_tile(const floatx16& s0, const floatx16
       const float x0 = ts < 2 ? s0[i] : s1[i], x1 = ts < 2 ? s0[i + 1] : s1[i + 1];
       const float p0 = __builtin_amdgcn_exp2f(FOLD ? x0 : __builtin_fmaf(x0, qk_scale, -m));
       const float p1 = __builtin_amdgcn_exp2f(FOLD ? x1 : __builtin_fmaf(x1, qk_scale, -m));
-      const half2v hp = {(_Float16)p0, (_Float16)p1};
-      l = __builtin_amdgcn_fdot2(hp, ones, l, false);
-      pf[ts][qb][jj] = __builtin_bit_cast(unsigned int, hp);
+      const unsigned int hp = pack2<PB>(p0, p1);
+      l = add_packed2<PB>(hp, l);
+      pf[ts][qb][jj] = hp;
     }
   }
   return l;

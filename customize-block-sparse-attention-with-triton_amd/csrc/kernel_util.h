@@ -39,6 +39,32 @@ __device__ __forceinline__ floatx16 mfma_qk(uintx4 a, uintx4 b, floatx16 c) {
                                                   __builtin_bit_cast(half8, b), c, 0, 0, 0);
 }
 
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// Two fp32 values rounded to the 16-bit type of the second products (PB: bf16, else fp16), packed.
+template <bool PB>
+__device__ __forceinline__ unsigned int pack2(float a, float b) {
+  if constexpr (PB) {
+    const bf16x2 h = {(__bf16)a, (__bf16)b};
+    return __builtin_bit_cast(unsigned int, h);
+  } else {
+    const half2v h = {(_Float16)a, (_Float16)b};
+    return __builtin_bit_cast(unsigned int, h);
+  }
+}
+
+// acc + the two packed 16-bit values of x (what a second product will see of them)
+template <bool PB>
+__device__ __forceinline__ float add_packed2(unsigned int x, float acc) {
+  if constexpr (PB) {
+    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, x), ones, acc, false);
+  } else {
+    const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, x), ones, acc, false);
+  }
+}
+
 // two packed fp16 values times an fp32 scalar, rounded back to fp16
 __device__ __forceinline__ unsigned int scale_half2(unsigned int x, float c) {
   const half2v h = __builtin_bit_cast(half2v, x);

@@ -142,3 +142,28 @@ def test_autograd_with_elementwise_mask(dev):
     fm.flash_attention_custom_mask(qd, kd, vd, mask.to(dev), 0.125).backward(do.to(dev))
     for got, ref in ((qd.grad, dq_r), (kd.grad, dk_r), (vd.grad, dv_r)):
         assert errors(got, ref)[0] <= 2e-2
+
+
+@pytest.mark.parametrize("D,B,H", [(64, 1, 2), (128, 1, 2), (128, 4, 64)])
+def test_bf16_typed_outputs_elementwise(dev, D, B, H):
+    """bf16 inputs with bf16-typed results (P and dS rounded to bf16, no tile converted): forward and
+    gradients with an elementwise mask against the oracle; the cast of an exact result to bf16 alone is
+    1.7e-3 in rel-L2, hence the 3e-3 bar.  (B, H) = (4, 64) takes the many-row-blocks forward at D = 128."""
+    import fa2_custom_mask as fm
+    g = torch.Generator().manual_seed(67)
+    N = 384
+    mask = (torch.rand(1, 1, N, N, generator=g) < 0.5) & token_causal(N)
+    mask[0, 0, 100, :] = False
+    q, k, v, do = make_qkv(B, H, N, D, torch.bfloat16, 68, n=4)
+    sc = 1.0 / np.sqrt(D)
+    hs = slice(0, 2)                                   # oracle on two heads of the first batch entry
+    o_r = orc.naive_attention(f32(q[:1, hs]), f32(k[:1, hs]), f32(v[:1, hs]), mask.numpy(), sc)
+    dq_r, dk_r, dv_r, _ = orc.attention_backward(f32(q[:1, hs]), f32(k[:1, hs]), f32(v[:1, hs]), mask.numpy(), sc,
+                                                 f32(do[:1, hs]))
+    o, lse, dq, dk, dv = fm.attention_forward_backward(q.to(dev), k.to(dev), v.to(dev), mask.to(dev), sc, do.to(dev))
+    torch.cuda.synchronize()
+    for name, got, ref in (("o", o, o_r), ("dq", dq, dq_r), ("dk", dk, dk_r), ("dv", dv, dv_r)):
+        assert got.dtype == torch.bfloat16
+        ma, rl = errors(got[:1, hs], ref)
+        print("%s D%d: max-abs %.3e rel-L2 %.3e" % (name, D, ma, rl))
+        assert ma <= 3e-2 and rl <= 3e-3, name
