@@ -71,23 +71,24 @@ __global__ __launch_bounds__(256) void delta_kernel(const BwdParams prm) {
 // ---------------------------------------------------------------------------------------
 // helpers of the two walking kernels
 // ---------------------------------------------------------------------------------------
-template <int D, bool EW> struct BwdCfg {
-  static constexpr int TILE_BYTES = 64 * 2 * D;
+// ROWS: rows of a tile staged per step (64, or 32 when a tile is walked in two halves)
+template <int D, bool EW, int ROWS = 64> struct BwdCfg {
+  static constexpr int TILE_BYTES = ROWS * 2 * D;
   static constexpr int STAT_BYTES = 2 * 64 * 4;                    // lse2[64] + delta[64] of a row block
   static constexpr int BITS_BYTES = EW ? 64 * 8 : 0;               // mask words of the tile (elementwise masks)
   static constexpr int STAGE_BYTES = 2 * TILE_BYTES + STAT_BYTES + BITS_BYTES;  // two tiles, row statistics, mask words
   static constexpr int LDS_BYTES = 2 * STAGE_BYTES;                // double buffer
 };
 
-// This wavefront's half of the asynchronous copy of a 64 x D tile (rows `stride` elements apart)
-// into LDS with the u_swz chunk swizzle: wavefront wv issues instructions [wv*D/16, (wv+1)*D/16).
-template <int D>
+// This wavefront's half of the asynchronous copy of a ROWS x D tile (rows `stride` elements apart)
+// into LDS with the u_swz chunk swizzle: wavefront wv issues half of the ROWS*D/512 instructions.
+template <int D, int ROWS = 64>
 __device__ __forceinline__ void half_tile_load_async(const unsigned short* tile, int64_t stride, int wv, int lane,
                                                      unsigned lds_addr) {
-  constexpr int CPR = D / 8;
+  constexpr int CPR = D / 8, PER_WAVE = ROWS * CPR / 128;
 #pragma unroll
-  for (int jj = 0; jj < CPR / 2; ++jj) {
-    const int j = wv * (CPR / 2) + jj;
+  for (int jj = 0; jj < PER_WAVE; ++jj) {
+    const int j = wv * PER_WAVE + jj;
     const int c = j * 64 + lane, row = c / CPR, ch = c % CPR;
     const unsigned off = 2u * (unsigned)(row * (int)stride + ((ch ^ u_swz<D>(row)) * 8));
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
@@ -140,6 +141,12 @@ __device__ __forceinline__ void mask_scores(floatx16& s0, floatx16& s1, unsigned
   }
 }
 
+// the same for one block of 32 keys (bits 0..31 of the shifted word)
+__device__ __forceinline__ void mask_scores(floatx16& s0, unsigned lo) {
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s0[i] = (lo & (1u << (8 * (i / 4) + (i % 4)))) ? s0[i] : -INFINITY;
+}
+
 __device__ __forceinline__ floatx16 zero16() {
   floatx16 z;
 #pragma unroll
@@ -164,10 +171,13 @@ __device__ __forceinline__ void head_and_block(int L, int BH, int nb, int& bh, i
 // ---------------------------------------------------------------------------------------
 // PB (bf16 inputs only): dS is rounded to bf16 and the second product runs in bf16 on the tile as it
 // is; otherwise dS is rounded to fp16 and bf16 tiles are converted fragment by fragment.
-template <int D, bool BF16, bool EW, bool PB>
-__global__ __launch_bounds__(128) void dq_kernel(const BwdParams prm) {
-  using C = BwdCfg<D, EW>;
-  constexpr int KS = D / 16, DB = D / 32;
+// KB: 32-key blocks of a tile handled per step.  2: a whole tile per step.  1 (used at D = 128): a
+// tile is walked in two steps of 32 keys; the staged halves are 8 KB, four workgroups fit a compute
+// unit and the wavefront stays within 256 registers: two wavefronts per SIMD.
+template <int D, bool BF16, bool EW, bool PB, int KB>
+__global__ __launch_bounds__(128, 2) void dq_kernel(const BwdParams prm) {
+  using C = BwdCfg<D, EW, 32 * KB>;
+  constexpr int KS = D / 16, DB = D / 32, STEPS = 2 / KB;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int ln = lane & 31, g = lane >> 5;
@@ -180,21 +190,22 @@ __global__ __launch_bounds__(128) void dq_kernel(const BwdParams prm) {
   const int mh = (prm.Bm > 1 ? b : 0) * prm.Hm + (prm.Hm > 1 ? h : 0);
   const cint_ptr_t rp = (cint_ptr_t)(uintptr_t)(prm.row_ptr + (int64_t)mh * nb);
   const cint_ptr_t cols = (cint_ptr_t)(uintptr_t)prm.col_idx;
-  const int t0 = rp[m], t1 = rp[m + 1];
+  const int u0 = rp[m] * STEPS, u1 = rp[m + 1] * STEPS;       // steps: tile u / STEPS, part u % STEPS
   const unsigned lds_addr = (unsigned)(uintptr_t)(lds_ptr_t)lds;
 
   const unsigned short* kg = (const unsigned short*)prm.k + b * prm.ks[0] + h * prm.ks[1];
   const unsigned short* vg = (const unsigned short*)prm.v + b * prm.vs[0] + h * prm.vs[1];
-  auto issue = [&](int t, int stage) {
-    const int cb = cols[t];
-    half_tile_load_async<D>(kg + (int64_t)cb * 64 * prm.ks[2], prm.ks[2], wv, lane, lds_addr + stage * C::STAGE_BYTES);
-    half_tile_load_async<D>(vg + (int64_t)cb * 64 * prm.vs[2], prm.vs[2], wv, lane,
-                            lds_addr + stage * C::STAGE_BYTES + C::TILE_BYTES);
+  auto issue = [&](int u, int stage) {
+    const int t = u / STEPS;
+    const int64_t key0 = (int64_t)cols[t] * 64 + (u % STEPS) * 32 * KB;
+    half_tile_load_async<D, 32 * KB>(kg + key0 * prm.ks[2], prm.ks[2], wv, lane, lds_addr + stage * C::STAGE_BYTES);
+    half_tile_load_async<D, 32 * KB>(vg + key0 * prm.vs[2], prm.vs[2], wv, lane,
+                                     lds_addr + stage * C::STAGE_BYTES + C::TILE_BYTES);
     if constexpr (EW)   // the tile's 64 mask words, 256 bytes per wavefront
       stat_load_async(reinterpret_cast<const float*>(prm.bits_rows + (int64_t)t * 64) + wv * 64, lane,
                       lds_addr + stage * C::STAGE_BYTES + 2 * C::TILE_BYTES + C::STAT_BYTES + wv * 256);
   };
-  if (t0 < t1) issue(t0, 0);
+  if (u0 < u1) issue(u0, 0);
 
   const int64_t qrow = (int64_t)m * 64 + 32 * wv + ln;
   const unsigned short* qp = (const unsigned short*)prm.q + b * prm.qs[0] + h * prm.qs[1] + qrow * prm.qs[2];
@@ -217,52 +228,55 @@ __global__ __launch_bounds__(128) void dq_kernel(const BwdParams prm) {
 #pragma unroll
   for (int db = 0; db < DB; ++db) dqacc[db] = zero16();
 
-  for (int t = t0; t < t1; ++t) {
-    const int stage = (t - t0) & 1;
+  for (int u = u0; u < u1; ++u) {
+    const int stage = (u - u0) & 1;
     wait_vm<0>();
-    __syncthreads();   // tile t complete in `stage`; everyone is done with the other stage
-    if (t + 1 < t1) issue(t + 1, stage ^ 1);
+    __syncthreads();   // step u complete in `stage`; everyone is done with the other stage
+    if (u + 1 < u1) issue(u + 1, stage ^ 1);
     const unsigned char* kt = lds + stage * C::STAGE_BYTES;
     const unsigned char* vt = kt + C::TILE_BYTES;
 
     // All operand fragments of a block of MFMAs are read from LDS before the block starts: a read
     // issued next to the MFMA that consumes it costs a full LDS latency per MFMA.
-    uintx4 fk[2][KS], fv[2][KS];
+    uintx4 fk[KB][KS], fv[KB][KS];
 #pragma unroll
     for (int s = 0; s < KS; ++s)
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
+      for (int kb = 0; kb < KB; ++kb) {
         fk[kb][s] = frag_rows<D>(kt, 32 * kb, s, ln, g);
         fv[kb][s] = frag_rows<D>(vt, 32 * kb, s, ln, g);
       }
     __builtin_amdgcn_sched_barrier(0);
-    floatx16 sacc[2], dpacc[2];
+    floatx16 sacc[KB], dpacc[KB];
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) { sacc[kb] = zero16(); dpacc[kb] = zero16(); }
+    for (int kb = 0; kb < KB; ++kb) { sacc[kb] = zero16(); dpacc[kb] = zero16(); }
 #pragma unroll
     for (int s = 0; s < KS; ++s)
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
+      for (int kb = 0; kb < KB; ++kb) {
         sacc[kb] = mfma_qk<BF16>(fk[kb][s], qfr[s], sacc[kb]);      // S^T = K Q^T
         dpacc[kb] = mfma_qk<BF16>(fv[kb][s], dofr[s], dpacc[kb]);   // dP^T = V dO^T
       }
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (EW) {
-      const unsigned long long mw = *reinterpret_cast<const unsigned long long*>(
-          vt + C::TILE_BYTES + C::STAT_BYTES + (32 * wv + ln) * 8) >> (4 * g);
-      mask_scores(sacc[0], sacc[1], mw);
+      unsigned long long mw = *reinterpret_cast<const unsigned long long*>(
+          vt + C::TILE_BYTES + C::STAT_BYTES + (32 * wv + ln) * 8);
+      if constexpr (KB == 1) mw >>= 32 * (u % STEPS);
+      mw >>= 4 * g;
+      if constexpr (KB == 2) mask_scores(sacc[0], sacc[1], mw);
+      else mask_scores(sacc[0], (unsigned)mw);
     }
     // K^T fragments of the second product, read under the exponentials below
-    uintx4 fkt[4][DB];
+    uintx4 fkt[2 * KB][DB];
 #pragma unroll
-    for (int ts = 0; ts < 4; ++ts)
+    for (int ts = 0; ts < 2 * KB; ++ts)
 #pragma unroll
       for (int db = 0; db < DB; ++db) fkt[ts][db] = frag_cols<D, BF16 && !PB>(kt, db, ts, lane);
     __builtin_amdgcn_sched_barrier(0);
     // dS^T = P^T * (dP^T - delta), this lane's query; packed as operand slices of 16 keys
-    uintx4 dsf[4];
+    uintx4 dsf[2 * KB];
 #pragma unroll
-    for (int ts = 0; ts < 4; ++ts)
+    for (int ts = 0; ts < 2 * KB; ++ts)
 #pragma unroll
       for (int jj = 0; jj < 4; ++jj) {
         const int kb = ts >> 1, i = 8 * (ts & 1) + 2 * jj;
@@ -271,7 +285,7 @@ __global__ __launch_bounds__(128) void dq_kernel(const BwdParams prm) {
         dsf[ts][jj] = pack2<PB>(p0 * (dpacc[kb][i] - dlt), p1 * (dpacc[kb][i + 1] - dlt));
       }
 #pragma unroll
-    for (int ts = 0; ts < 4; ++ts)
+    for (int ts = 0; ts < 2 * KB; ++ts)
 #pragma unroll
       for (int db = 0; db < DB; ++db)
         dqacc[db] = mfma_qk<PB>(fkt[ts][db], dsf[ts], dqacc[db]);       // dQ^T += K^T dS^T
@@ -442,10 +456,12 @@ size_t bwd_workspace_bytes(int B, int H, int N, int D) {
 template <int D, bool BF16, bool EW, bool PB>
 static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
   using C = BwdCfg<D, EW>;
+  constexpr int KB = D == 128 ? 1 : 2;          // dq_kernel walks D = 128 tiles in two halves
+  using CQ = BwdCfg<D, EW, 32 * KB>;
   static bool configured = false;   // raising the dynamic LDS limit is idempotent
   if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dq_kernel<D, BF16, EW, PB>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dq_kernel<D, BF16, EW, PB, KB>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, CQ::LDS_BYTES);
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv_kernel<D, BF16, EW, PB>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
     configured = true;
@@ -454,7 +470,7 @@ static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
   constexpr int RPB = 256 / (D / 8);
   hipLaunchKernelGGL((delta_kernel<D, BF16>), dim3((prm.N + RPB - 1) / RPB, BH), dim3(256), 0, st, prm);
   const int grid = ((BH + 7) / 8) * 8 * prm.nb;   // heads in groups of 8, the last group padded
-  hipLaunchKernelGGL((dq_kernel<D, BF16, EW, PB>), dim3(grid), dim3(128), C::LDS_BYTES, st, prm);
+  hipLaunchKernelGGL((dq_kernel<D, BF16, EW, PB, KB>), dim3(grid), dim3(128), CQ::LDS_BYTES, st, prm);
   hipLaunchKernelGGL((dkdv_kernel<D, BF16, EW, PB>), dim3(grid), dim3(128), C::LDS_BYTES, st, prm);
 }
 
