@@ -304,10 +304,12 @@ __global__ __launch_bounds__(128, 2) void dq_kernel(const BwdParams prm) {
 // ---------------------------------------------------------------------------------------
 // dK, dV: workgroup = column block n, wavefront wv owns keys 64n + 32wv + ln
 // ---------------------------------------------------------------------------------------
-template <int D, bool BF16, bool EW, bool PB>
+// QB: 32-query blocks of a tile handled per step (2: a whole tile; 1: a tile in two halves, which
+// halves the fragments in flight).
+template <int D, bool BF16, bool EW, bool PB, int QB>
 __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
-  using C = BwdCfg<D, EW>;
-  constexpr int KS = D / 16, DB = D / 32;
+  using C = BwdCfg<D, EW, 32 * QB>;
+  constexpr int KS = D / 16, DB = D / 32, STEPS = 2 / QB;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int ln = lane & 31, g = lane >> 5;
@@ -319,24 +321,26 @@ __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
   const int mh = (prm.Bm > 1 ? b : 0) * prm.Hm + (prm.Hm > 1 ? h : 0);
   const cint_ptr_t cp = (cint_ptr_t)(uintptr_t)(prm.col_ptr + (int64_t)mh * nb);
   const cint_ptr_t rows = (cint_ptr_t)(uintptr_t)prm.row_idx;
-  const int t0 = cp[n], t1 = cp[n + 1];
+  const int u0 = cp[n] * STEPS, u1 = cp[n + 1] * STEPS;        // steps: tile u / STEPS, part u % STEPS
   const unsigned lds_addr = (unsigned)(uintptr_t)(lds_ptr_t)lds;
 
   const unsigned short* qg = (const unsigned short*)prm.q + b * prm.qs[0] + h * prm.qs[1];
   const unsigned short* gg = (const unsigned short*)prm.d_o + b * prm.dos[0] + h * prm.dos[1];
   const float* lse_h = prm.lse + (int64_t)bh * prm.N;
   const float* dlt_h = prm.delta + (int64_t)bh * prm.N;
-  auto issue = [&](int t, int stage) {
+  auto issue = [&](int u, int stage) {
+    const int t = u / STEPS;
     const int rb = rows[t];
+    const int64_t row0 = (int64_t)rb * 64 + (u % STEPS) * 32 * QB;
     const unsigned sa = lds_addr + stage * C::STAGE_BYTES;
-    half_tile_load_async<D>(qg + (int64_t)rb * 64 * prm.qs[2], prm.qs[2], wv, lane, sa);
-    half_tile_load_async<D>(gg + (int64_t)rb * 64 * prm.dos[2], prm.dos[2], wv, lane, sa + C::TILE_BYTES);
-    stat_load_async((wv == 0 ? lse_h : dlt_h) + rb * 64, lane, sa + 2 * C::TILE_BYTES + wv * 256);
+    half_tile_load_async<D, 32 * QB>(qg + row0 * prm.qs[2], prm.qs[2], wv, lane, sa);
+    half_tile_load_async<D, 32 * QB>(gg + row0 * prm.dos[2], prm.dos[2], wv, lane, sa + C::TILE_BYTES);
+    stat_load_async((wv == 0 ? lse_h : dlt_h) + rb * 64, lane, sa + 2 * C::TILE_BYTES + wv * 256);   // all 64 rows of the tile
     if constexpr (EW)   // the tile's 64 mask words (one per key, bit = query), 256 bytes per wavefront
       stat_load_async(reinterpret_cast<const float*>(prm.bits_cols + (int64_t)t * 64) + wv * 64, lane,
                       sa + 2 * C::TILE_BYTES + C::STAT_BYTES + wv * 256);
   };
-  if (t0 < t1) issue(t0, 0);
+  if (u0 < u1) issue(u0, 0);
 
   const int64_t krow = (int64_t)n * 64 + 32 * wv + ln;
   const unsigned short* kp = (const unsigned short*)prm.k + b * prm.ks[0] + h * prm.ks[1] + krow * prm.ks[2];
@@ -354,46 +358,50 @@ __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
 #pragma unroll
   for (int db = 0; db < DB; ++db) { dkacc[db] = zero16(); dvacc[db] = zero16(); }
 
-  for (int t = t0; t < t1; ++t) {
-    const int stage = (t - t0) & 1;
+  for (int u = u0; u < u1; ++u) {
+    const int stage = (u - u0) & 1;
     wait_vm<0>();
     __syncthreads();
-    if (t + 1 < t1) issue(t + 1, stage ^ 1);
+    if (u + 1 < u1) issue(u + 1, stage ^ 1);
     const unsigned char* qt = lds + stage * C::STAGE_BYTES;
     const unsigned char* gt = qt + C::TILE_BYTES;
-    const float* st_lse = reinterpret_cast<const float*>(gt + C::TILE_BYTES);
+    const int qoff = QB == 1 ? 32 * (u % STEPS) : 0;            // first query of this step within the tile
+    const float* st_lse = reinterpret_cast<const float*>(gt + C::TILE_BYTES) + qoff;
     const float* st_dlt = st_lse + 64;
 
     // operand fragments are read from LDS ahead of the block of MFMAs that consumes them
-    uintx4 fq[2][KS], fg[2][KS];
+    uintx4 fq[QB][KS], fg[QB][KS];
 #pragma unroll
     for (int s = 0; s < KS; ++s)
 #pragma unroll
-      for (int qb = 0; qb < 2; ++qb) {
+      for (int qb = 0; qb < QB; ++qb) {
         fq[qb][s] = frag_rows<D>(qt, 32 * qb, s, ln, g);
         fg[qb][s] = frag_rows<D>(gt, 32 * qb, s, ln, g);
       }
     __builtin_amdgcn_sched_barrier(0);
-    floatx16 sacc[2], dpacc[2];
+    floatx16 sacc[QB], dpacc[QB];
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb) { sacc[qb] = zero16(); dpacc[qb] = zero16(); }
+    for (int qb = 0; qb < QB; ++qb) { sacc[qb] = zero16(); dpacc[qb] = zero16(); }
 #pragma unroll
     for (int s = 0; s < KS; ++s)
 #pragma unroll
-      for (int qb = 0; qb < 2; ++qb) {
+      for (int qb = 0; qb < QB; ++qb) {
         sacc[qb] = mfma_qk<BF16>(fq[qb][s], kfr[s], sacc[qb]);      // S = Q K^T
         dpacc[qb] = mfma_qk<BF16>(fg[qb][s], vfr[s], dpacc[qb]);    // dP = dO V^T
       }
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (EW) {
-      const unsigned long long mw = *reinterpret_cast<const unsigned long long*>(
-          gt + C::TILE_BYTES + C::STAT_BYTES + (32 * wv + ln) * 8) >> (4 * g);
-      mask_scores(sacc[0], sacc[1], mw);
+      unsigned long long mw = *reinterpret_cast<const unsigned long long*>(
+          gt + C::TILE_BYTES + C::STAT_BYTES + (32 * wv + ln) * 8);
+      if constexpr (QB == 1) mw >>= qoff;
+      mw >>= 4 * g;
+      if constexpr (QB == 2) mask_scores(sacc[0], sacc[1], mw);
+      else mask_scores(sacc[0], (unsigned)mw);
     }
     // dO^T and Q^T fragments of the second products, read under the exponentials below
-    uintx4 fgt[4][DB], fqt[4][DB];
+    uintx4 fgt[2 * QB][DB], fqt[2 * QB][DB];
 #pragma unroll
-    for (int ts = 0; ts < 4; ++ts)
+    for (int ts = 0; ts < 2 * QB; ++ts)
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         fgt[ts][db] = frag_cols<D, BF16 && !PB>(gt, db, ts, lane);
@@ -401,9 +409,9 @@ __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
       }
     __builtin_amdgcn_sched_barrier(0);
     // rows of the results are queries: register i of block qb <-> query 32qb + 8(i/4) + 4g + i%4
-    uintx4 pf[4], dsf[4];
+    uintx4 pf[2 * QB], dsf[2 * QB];
 #pragma unroll
-    for (int ts = 0; ts < 4; ++ts)
+    for (int ts = 0; ts < 2 * QB; ++ts)
 #pragma unroll
       for (int jh = 0; jh < 2; ++jh) {
         const int qb = ts >> 1, i0 = 8 * (ts & 1) + 4 * jh;
@@ -422,7 +430,7 @@ __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
         dsf[ts][2 * jh] = pack2<PB>(ds[0], ds[1]); dsf[ts][2 * jh + 1] = pack2<PB>(ds[2], ds[3]);
       }
 #pragma unroll
-    for (int ts = 0; ts < 4; ++ts)
+    for (int ts = 0; ts < 2 * QB; ++ts)
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         dvacc[db] = mfma_qk<PB>(fgt[ts][db], pf[ts], dvacc[db]);    // dV^T += dO^T P
@@ -458,12 +466,15 @@ static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
   using C = BwdCfg<D, EW>;
   constexpr int KB = D == 128 ? 1 : 2;          // dq_kernel walks D = 128 tiles in two halves
   using CQ = BwdCfg<D, EW, 32 * KB>;
+  constexpr int QB = 2;   // dkdv_kernel keeps one wavefront per SIMD either way (K, V, dK, dV of 32 keys are 192
+                          // registers at D = 128); halves were measured slower there (718 against 688 us, C5)
+  using CK = BwdCfg<D, EW, 32 * QB>;
   static bool configured = false;   // raising the dynamic LDS limit is idempotent
   if (!configured) {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dq_kernel<D, BF16, EW, PB, KB>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, CQ::LDS_BYTES);
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv_kernel<D, BF16, EW, PB>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv_kernel<D, BF16, EW, PB, QB>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, CK::LDS_BYTES);
     configured = true;
   }
   const int BH = prm.B * prm.H;
@@ -471,7 +482,7 @@ static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
   hipLaunchKernelGGL((delta_kernel<D, BF16>), dim3((prm.N + RPB - 1) / RPB, BH), dim3(256), 0, st, prm);
   const int grid = ((BH + 7) / 8) * 8 * prm.nb;   // heads in groups of 8, the last group padded
   hipLaunchKernelGGL((dq_kernel<D, BF16, EW, PB, KB>), dim3(grid), dim3(128), CQ::LDS_BYTES, st, prm);
-  hipLaunchKernelGGL((dkdv_kernel<D, BF16, EW, PB>), dim3(grid), dim3(128), C::LDS_BYTES, st, prm);
+  hipLaunchKernelGGL((dkdv_kernel<D, BF16, EW, PB, QB>), dim3(grid), dim3(128), CK::LDS_BYTES, st, prm);
 }
 
 int launch_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
