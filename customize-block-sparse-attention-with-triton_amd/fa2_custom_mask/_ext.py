@@ -4,6 +4,7 @@ There is deliberately no fallback: if the library is missing, or a call returns 
 code, a RuntimeError is raised.
 """
 import ctypes
+import functools
 import os
 
 import torch
@@ -67,26 +68,35 @@ def dtype_code(dt):
         raise TypeError("unsupported dtype %s" % dt)
 
 
+@functools.lru_cache(maxsize=256)
+def _strides_array(strides):
+    return (ctypes.c_int64 * 4)(*strides)
+
+
 def strides4(t):
-    return (ctypes.c_int64 * 4)(*t.stride())
+    """Element strides of a 4-d tensor as a C array (cached per stride tuple; never written to)."""
+    return _strides_array(t.stride())
 
 
 def current_stream(device):
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
+@functools.lru_cache(maxsize=256)
 def mask_lists_workspace(Bm, Hm, nb):
     n = ctypes.c_size_t()
     check(lib().bsattn_mask_lists_workspace(Bm, Hm, nb, ctypes.byref(n)), "bsattn_mask_lists_workspace")
     return n.value
 
 
+@functools.lru_cache(maxsize=256)
 def fwd_workspace(B, H, N, D):
     n = ctypes.c_size_t()
     check(lib().bsattn_fwd_workspace(B, H, N, D, ctypes.byref(n)), "bsattn_fwd_workspace")
     return n.value
 
 
+@functools.lru_cache(maxsize=256)
 def bwd_workspace(B, H, N, D):
     n = ctypes.c_size_t()
     check(lib().bsattn_bwd_workspace(B, H, N, D, ctypes.byref(n)), "bsattn_bwd_workspace")
