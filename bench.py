@@ -96,6 +96,35 @@ def elementwise_case(torch, dev, fm, q, k, v, sm_scale):
             "preprocess_ms": round(tp[len(tp) // 2], 5), "max_abs_vs_torch_fp32": err}
 
 
+def reorder_case(torch, dev, fm):
+    """Head-wise token reorder and its inverse (the step either side of attention in the caller) at the
+    reference's default video shape, functional.py:22: F, H, W = 13, 30, 45 (17 550 tokens), 48 heads of
+    64 fp16 values.  HBM bound: bytes = read + write of the tensor."""
+    F, H, W, heads, D = 13, 30, 45, 48, 64
+    g = torch.Generator().manual_seed(SEED + 9)
+    x = torch.randn(1, heads, F * H * W, D, generator=g).to(torch.float16).to(dev)
+    perms = torch.tensor([[0, 1, 2], [0, 2, 1], [1, 2, 0], [1, 0, 2], [2, 1, 0], [2, 0, 1]], dtype=torch.int32)
+    invs = torch.tensor([[0, 1, 2], [0, 2, 1], [2, 0, 1], [1, 0, 2], [2, 1, 0], [1, 2, 0]], dtype=torch.int32)
+    idx = torch.arange(heads) % 6
+    orders, inv_orders = perms[idx].to(dev), invs[idx].to(dev)
+    y = fm.apply_head_wise_reorder(x, orders, F, H, W)
+    back = fm.apply_inv_reorder(y, orders, inv_orders, F, H, W)
+    ok = bool(torch.equal(back, x))
+    # closed form of one head: view as (F, H, W), permute, flatten (permute.py:45-58)
+    hd = 5
+    ref = x[0, hd].view(F, H, W, D).permute(*perms[idx[hd]].tolist(), 3).reshape(F * H * W, D)
+    ok = ok and bool(torch.equal(y[0, hd], ref))
+    tf = event_times(lambda: fm.apply_head_wise_reorder(x, orders, F, H, W), 20, 3, torch)
+    ti = event_times(lambda: fm.apply_inv_reorder(y, orders, inv_orders, F, H, W), 20, 3, torch)
+    nbytes = 2.0 * x.numel() * x.element_size()
+    mf, mi = tf[len(tf) // 2], ti[len(ti) // 2]
+    return {"workload": "reorder + inverse, 1 x 48 heads x 17550 tokens x 64 fp16 (F,H,W = 13,30,45)",
+            "bytes": nbytes, "reorder_ms": round(mf, 5), "inverse_ms": round(mi, 5),
+            "reorder_GBps": round(nbytes / mf / 1e6, 1), "inverse_GBps": round(nbytes / mi / 1e6, 1),
+            "frac_hbm_peak": round(nbytes / mf / 1e6 / PEAK_HBM_GBS, 4), "bit_exact_round_trip_and_closed_form": ok,
+            "note": "times include the output allocation of the host wrapper"}
+
+
 def mfma_ceiling(torch, dev, iters=8192, launches=10):
     """Sustained fp16 MFMA rate (TFLOP/s) of bsattn_mfma_rate_probe for two operand patterns."""
     import ctypes
@@ -134,6 +163,8 @@ def main():
     ap.add_argument("--fwd-bwd", action="store_true",
                     help="measurement aid: forward and backward at BASELINE configs[4] (B=2 H=16 N=8192 D=128 bf16, "
                          "block-causal mask with keep 0.25 shared by all heads), then exit")
+    ap.add_argument("--reorder", action="store_true",
+                    help="measurement aid: the head-wise token reorder and its inverse, then exit")
     ap.add_argument("--mfma-ceiling", action="store_true",
                     help="measurement aid: the fp16 MFMA rate the GPU sustains with all-ones operands and "
                          "with random operands (the clock depends on the data), then exit")
@@ -160,6 +191,9 @@ def main():
         return
     if args.mfma_ceiling:
         print(json.dumps(mfma_ceiling(torch, dev)))
+        return
+    if args.reorder:
+        print(json.dumps(reorder_case(torch, dev, fm)))
         return
     if args.fwd_bwd:
         print(json.dumps(fwd_bwd_c5(torch, dev, fm, min(args.steps, 50), min(args.warmup, 5))))
@@ -254,6 +288,7 @@ def main():
         "data_dependence": data_dependence,
         "fwd_bwd_configs4": fwd_bwd_c5(torch, dev, fm, 20, 3),
         "elementwise_mask": elementwise_case(torch, dev, fm, qd, kd, vd, sm_scale),
+        "token_reorder": reorder_case(torch, dev, fm),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
                      "kernel": "fwd_kernel<64, 0, false, false> (fp16, one bsattn_fwd call)",
