@@ -68,7 +68,9 @@ __device__ __forceinline__ void recentre(floatx16& s0, floatx16& s1, floatx16 (&
   float delta = fresh ? smax : fmaxf(smax, 0.f);
   bool nomass = false;
   if constexpr (EW) {
-    nomass = !fresh && l == 0.f;
+    // (a query's keys are split over two lanes, which must keep one common reference: the mass is
+    // the sum of both halves, or a lane whose own keys were all masked would drift away)
+    nomass = !fresh && l + __shfl_xor(l, 32) == 0.f;
     if (nomass) delta = smax;
     if (smax == -INFINITY) delta = 0.f;
   }

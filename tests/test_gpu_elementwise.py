@@ -167,3 +167,25 @@ def test_bf16_typed_outputs_elementwise(dev, D, B, H):
         ma, rl = errors(got[:1, hs], ref)
         print("%s D%d: max-abs %.3e rel-L2 %.3e" % (name, D, ma, rl))
         assert ma <= 3e-2 and rl <= 3e-3, name
+
+
+def test_large_scores_with_half_masked_queries_many_heads(dev):
+    """A query's 64 keys of a tile sit in two lanes.  With large score differences one lane's share of P can
+    round to zero while the other lane holds all the mass: both must still follow one reference
+    exponent.  Many heads, so that a wavefront walks whole row blocks (several tiles in a row)."""
+    g = torch.Generator().manual_seed(69)
+    N = 1024
+    m = torch.rand(1, 1, N, N, generator=g) < 0.3
+    m[0, 0, ::2, :448] = False
+    q, k, v = make_qkv(1, 1, N, 64, torch.float16, 70)
+    q = (q.float() * 8.0).to(torch.float16)
+    o_ref, lse_ref = orc.naive_attention(f32(q), f32(k), f32(v), m.numpy(), 0.125, return_lse=True)
+    import fa2_custom_mask as fm
+    H = 256
+    qq, kk, vv = [x.expand(1, H, N, 64).contiguous().to(dev) for x in (q, k, v)]
+    o, lse = fm.flash_attention_custom_mask_lse(qq, kk, vv, m.to(dev), 0.125, out_fp32=True)
+    torch.cuda.synchronize()
+    for hd in (0, 100, 255):
+        ma, rl = errors(o[:, hd:hd + 1], o_ref)
+        assert ma <= 2e-2 and rl <= 1e-3
+        assert np.abs(lse[:, hd:hd + 1].cpu().numpy() - lse_ref).max() <= 2e-2
