@@ -57,6 +57,10 @@ template <int D> struct FwdCfg {
   static constexpr int ROUNDS = D / R;
   static constexpr int QPW = (R / 4) / NW;                  // output quads per wavefront and round
   static constexpr int SHORT_ROW = 6 * NW;                  // row blocks up to this many tiles may go to one wavefront
+#ifndef SNAP_TILES
+#define SNAP_TILES 8
+#endif
+  static constexpr int SNAP = SNAP_TILES;                   // a range boundary this close to an end of its row block moves there
 };
 
 // DT: 0 fp16; 1 bf16 with P rounded to fp16 (V fragments converted); 2 bf16 with P rounded to bf16.
@@ -86,15 +90,15 @@ void fwd_kernel(const FwdParams prm) {
   // the lists are read-only for the whole launch: constant address space => scalar loads
   const cint_ptr_t rp = (cint_ptr_t)(uintptr_t)(prm.row_ptr + (int64_t)mh * nb);
   const cint_ptr_t cols = (cint_ptr_t)(uintptr_t)prm.col_idx;
-  const HeadSplit hs = head_split(rp, nb, prm.W, NW, prm.first_ids > bh ? (prm.first_ids - bh + BH - 1) / BH : 0);
-  // a head without kept tiles still needs its zeros: workgroup 0 writes them
-  const int Pact = hs.T == 0 ? 1 : hs.Peff;
-  if (wg >= Pact) return;
-  const int g0 = hs.T > 0 ? split_begin(hs, wg) : hs.lo, g1 = hs.T > 0 ? split_begin(hs, wg + 1) : hs.lo;
-  if constexpr (!ROWS) {
-    // Row blocks without kept tiles belong to no range: they are dealt round-robin, and the
-    // workgroup writes O = 0, lse = -inf for its share.
-    for (int r0 = wg; r0 < nb; r0 += Pact) {
+  #ifndef MIN_TILES
+#define MIN_TILES NW
+#endif
+  const HeadSplit hs = head_split(rp, nb, prm.W, MIN_TILES, prm.first_ids > bh ? (prm.first_ids - bh + BH - 1) / BH : 0);
+  // Row blocks without kept tiles belong to no range: they are dealt round-robin over all workgroups
+  // of the head, which write O = 0, lse = -inf for their share.  (With whole row blocks per
+  // wavefront the ranges are row-aligned and cover them, unless the head keeps nothing at all.)
+  if (!ROWS || hs.T == 0) {
+    for (int r0 = wg; r0 < nb; r0 += prm.W) {
       if (rp[r0 + 1] > rp[r0]) continue;
       void* ob = out_base(prm, b, h);
       for (int i = threadIdx.x; i < 64 * (D / 4); i += NW * 64) {
@@ -103,6 +107,10 @@ void fwd_kernel(const FwdParams prm) {
       }
       if (prm.lse != nullptr && threadIdx.x < 64) prm.lse[(int64_t)bh * prm.N + (int64_t)r0 * 64 + threadIdx.x] = -INFINITY;
     }
+  }
+  if (hs.T == 0 || wg >= hs.Peff) return;
+  int g0 = split_begin(hs, wg), g1 = split_begin(hs, wg + 1);
+  if constexpr (!ROWS) {
     if (g0 >= g1) return;
   }
 
@@ -349,16 +357,19 @@ void fwd_kernel(const FwdParams prm) {
   // Number of entries r in [0, nb] with rp[r] <= x, for two values of x at once.  The row pointers
   // ascend, so this is a search; it is done in two rounds of one load per lane (64 evenly spaced
   // entries, then the entries between two of them) instead of a chain of dependent scalar loads.
-  auto count_le2 = [&](int x0, int x1, int& c0, int& c1) {
+  // Also returns the entries around x: s = rp[c - 1] (the last one <= x) and e = rp[c] (c <= nb).
+  auto count_le2 = [&](int x0, int x1, int& c0, int& c1, int& s0, int& e0, int& s1, int& e1) {
     const int32_t* rpg_ = prm.row_ptr + (int64_t)mh * nb;
     const int step = (nb + 64) / 64;
-    if (step > 64) {     // very long sequences: plain binary searches
+    if (step >= 64) {     // very long sequences: plain binary searches
       int lo = -1, hi = nb + 1;
       while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (rp[mid] <= x0) lo = mid; else hi = mid; }
       c0 = hi;
       lo = -1; hi = nb + 1;
       while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (rp[mid] <= x1) lo = mid; else hi = mid; }
       c1 = hi;
+      s0 = c0 > 0 ? rp[c0 - 1] : 0; e0 = c0 <= nb ? rp[c0] : 0x7fffffff;
+      s1 = c1 > 0 ? rp[c1 - 1] : 0; e1 = c1 <= nb ? rp[c1] : 0x7fffffff;
       return;
     }
     const int i1 = lane * step;
@@ -366,10 +377,15 @@ void fwd_kernel(const FwdParams prm) {
     const int a0 = __builtin_popcountll(__ballot(v1 <= x0)), a1 = __builtin_popcountll(__ballot(v1 <= x1));
     const int b0 = (a0 > 0 ? a0 - 1 : 0) * step, b1 = (a1 > 0 ? a1 - 1 : 0) * step;
     const int j0 = b0 + lane, j1 = b1 + lane;
-    const int w0 = lane < step && j0 <= nb ? rpg_[j0] : 0x7fffffff;
-    const int w1 = lane < step && j1 <= nb ? rpg_[j1] : 0x7fffffff;
-    c0 = a0 > 0 ? b0 + __builtin_popcountll(__ballot(w0 <= x0)) : 0;
-    c1 = a1 > 0 ? b1 + __builtin_popcountll(__ballot(w1 <= x1)) : 0;
+    // (lane `step` holds the next evenly spaced entry, which is > x: it does not count, but may be e)
+    const int w0 = lane <= step && j0 <= nb ? rpg_[j0] : 0x7fffffff;
+    const int w1 = lane <= step && j1 <= nb ? rpg_[j1] : 0x7fffffff;
+    const int k0 = a0 > 0 ? __builtin_popcountll(__ballot(w0 <= x0)) : 0;
+    const int k1 = a1 > 0 ? __builtin_popcountll(__ballot(w1 <= x1)) : 0;
+    c0 = b0 + k0;
+    c1 = b1 + k1;
+    s0 = __builtin_amdgcn_readfirstlane(__shfl(w0, k0 > 0 ? k0 - 1 : 0)); e0 = __builtin_amdgcn_readfirstlane(__shfl(w0, k0));
+    s1 = __builtin_amdgcn_readfirstlane(__shfl(w1, k1 > 0 ? k1 - 1 : 0)); e1 = __builtin_amdgcn_readfirstlane(__shfl(w1, k1));
   };
 
   int* ctr = reinterpret_cast<int*>(ml + NW * 2 * 64);
@@ -470,7 +486,8 @@ void fwd_kernel(const FwdParams prm) {
     int r_lo, r_hi;
     {
       // smallest r with rp[r] >= g = number of r with rp[r] <= g - 1 (capped at nb)
-      count_le2(g0 - 1, g1 - 1, r_lo, r_hi);
+      int u0, u1, u2, u3;
+      count_le2(g0 - 1, g1 - 1, r_lo, r_hi, u0, u1, u2, u3);
       r_lo = r_lo < nb ? r_lo : nb;
       r_hi = r_hi < nb ? r_hi : nb;
       if (wg >= hs.Peff - 1) r_hi = nb;    // trailing row blocks without kept tiles
@@ -492,11 +509,20 @@ void fwd_kernel(const FwdParams prm) {
     // K / V buffer has been issued; no copy is issued across the merge of a row block, which
     // borrows both buffers of every wavefront (one exchange round for the whole accumulator).
     // first row block of the range: largest r with rp[r] <= g0 < rp[r+1]
+    // A range boundary within SNAP tiles of an end of the row block it falls in moves to that end
+    // (the nearer one): sharing a row block costs a merge, a published part and a pull, several
+    // tiles' worth each, and row blocks of up to 2 SNAP tiles are never shared.  Every workgroup
+    // applies the same rule to both of its boundaries, so the ranges still tile the list.
     int r;
     {
-      int c0, c1;
-      count_le2(g0, g0, c0, c1);
+      int c0, c1, s0, e0, s1, e1;
+      count_le2(g0, g1, c0, c1, s0, e0, s1, e1);
       r = c0 - 1;
+      const int n0 = snap_boundary<C::SNAP>(g0, s0, e0);
+      if (n0 >= e0) ++r;
+      g0 = n0;
+      if (g1 < hs.lo + hs.T) g1 = snap_boundary<C::SNAP>(g1, s1, e1);
+      if (g0 >= g1) return;
     }
     stage_cols(g0, g1);
     if (threadIdx.x == 0) { ctr[0] = g0 + 2 * NW; ctr[3] = 0; }
@@ -679,7 +705,10 @@ void fwd_kernel(const FwdParams prm) {
             __hip_atomic_store(prm.flags + (int64_t)bh * prm.W + wg, prm.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         } else {
           // pull the parts of the workgroups wg+1 .. pl and finish the row block
-          const int pl_ = split_of_tile(hs, row_e - 1);
+          // (the last workgroup with tiles of this row block: a later one whose start moved to the row
+          // block's end holds none)
+          int pl_ = split_of_tile(hs, row_e - 1);
+          while (pl_ > wg && snap_boundary<C::SNAP>(split_begin(hs, pl_), row_s, row_e) >= row_e) --pl_;
           bool ok = true;
           for (int p = wg + 1; p <= pl_; ++p) {
             unsigned long long* fl = prm.flags + (int64_t)bh * prm.W + p;

@@ -51,4 +51,13 @@ __device__ __forceinline__ int split_of_tile(const HeadSplit& s, int t) {
 // floats per partial slot: unnormalised accumulator [64 x D] + running max [64] + sum [64]
 __host__ __device__ constexpr int partial_floats(int D) { return 64 * D + 128; }
 
+// Where a range boundary g inside the row block [s, e) of the tile list (s <= g < e) really goes: to
+// the nearer end of the row block if that is at most X tiles away, else it stays.
+template <int X>
+__device__ __forceinline__ int snap_boundary(int g, int s, int e) {
+  const int db = g - s, df = e - g;
+  if (db <= df) return db <= X ? s : g;
+  return df <= X ? e : g;
+}
+
 }  // namespace bsattn
