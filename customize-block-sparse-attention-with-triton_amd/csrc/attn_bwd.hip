@@ -29,6 +29,8 @@ struct BwdParams {
   const unsigned long long* bits_rows; const unsigned long long* bits_cols;
   int B, H, N, nb, Bm, Hm;
   int out_f32;
+  int split;                  // workgroups per row / column list (1: results written directly)
+  float* part_dq; float* part_dk; float* part_dv;   // split > 1: fp32 partial results [split][B*H][N][D]
   float sm_scale, qk_scale;   // qk_scale = sm_scale * log2(e)
   int64_t qs[3], ks[3], vs[3], os[3], dos[3];
 };
@@ -183,14 +185,21 @@ __global__ __launch_bounds__(128, 2) void dq_kernel(const BwdParams prm) {
   const int ln = lane & 31, g = lane >> 5;
   const int nb = prm.nb;
   int bh, blk;
-  head_and_block(blockIdx.x, prm.B * prm.H, nb, bh, blk);
+  const int per_chunk = gridDim.x / prm.split;               // chunk = slowest index: head i of a group stays on XCD i
+  const int chunk = blockIdx.x / per_chunk;
+  head_and_block(blockIdx.x - chunk * per_chunk, prm.B * prm.H, nb, bh, blk);
   if (blk >= nb) return;
   const int m = nb - 1 - blk;                 // long rows of block-causal masks first
   const int b = bh / prm.H, h = bh % prm.H;
   const int mh = (prm.Bm > 1 ? b : 0) * prm.Hm + (prm.Hm > 1 ? h : 0);
   const cint_ptr_t rp = (cint_ptr_t)(uintptr_t)(prm.row_ptr + (int64_t)mh * nb);
   const cint_ptr_t cols = (cint_ptr_t)(uintptr_t)prm.col_idx;
-  const int u0 = rp[m] * STEPS, u1 = rp[m + 1] * STEPS;       // steps: tile u / STEPS, part u % STEPS
+  int u0, u1;                                                  // steps: tile u / STEPS, part u % STEPS
+  {
+    const int t0 = rp[m], len = rp[m + 1] - t0;                // this workgroup's share of the row's list
+    u0 = (t0 + (int)((int64_t)len * chunk / prm.split)) * STEPS;
+    u1 = (t0 + (int)((int64_t)len * (chunk + 1) / prm.split)) * STEPS;
+  }
   const unsigned lds_addr = (unsigned)(uintptr_t)(lds_ptr_t)lds;
 
   const unsigned short* kg = (const unsigned short*)prm.k + b * prm.ks[0] + h * prm.ks[1];
@@ -291,6 +300,16 @@ __global__ __launch_bounds__(128, 2) void dq_kernel(const BwdParams prm) {
         dqacc[db] = mfma_qk<PB>(fkt[ts][db], dsf[ts], dqacc[db]);       // dQ^T += K^T dS^T
   }
 
+  if (prm.split > 1) {   // unscaled fp32 part; sum_parts_kernel adds the parts up
+    float* part = prm.part_dq + ((int64_t)chunk * prm.B * prm.H + bh) * prm.N * D;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4)
+        store_out4<BF16>(part, qrow * D + 32 * db + 8 * i4 + 4 * g, true, dqacc[db][4 * i4], dqacc[db][4 * i4 + 1],
+                         dqacc[db][4 * i4 + 2], dqacc[db][4 * i4 + 3]);
+    return;
+  }
   void* base = prm.out_f32 ? (void*)((float*)prm.dq + (int64_t)bh * prm.N * D) : (void*)((unsigned short*)prm.dq + (int64_t)bh * prm.N * D);
 #pragma unroll
   for (int db = 0; db < DB; ++db)
@@ -315,13 +334,20 @@ __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
   const int ln = lane & 31, g = lane >> 5;
   const int nb = prm.nb;
   int bh, n;                                  // early columns of block-causal masks are the long ones
-  head_and_block(blockIdx.x, prm.B * prm.H, nb, bh, n);
+  const int per_chunk = gridDim.x / prm.split;
+  const int chunk = blockIdx.x / per_chunk;
+  head_and_block(blockIdx.x - chunk * per_chunk, prm.B * prm.H, nb, bh, n);
   if (n >= nb) return;
   const int b = bh / prm.H, h = bh % prm.H;
   const int mh = (prm.Bm > 1 ? b : 0) * prm.Hm + (prm.Hm > 1 ? h : 0);
   const cint_ptr_t cp = (cint_ptr_t)(uintptr_t)(prm.col_ptr + (int64_t)mh * nb);
   const cint_ptr_t rows = (cint_ptr_t)(uintptr_t)prm.row_idx;
-  const int u0 = cp[n] * STEPS, u1 = cp[n + 1] * STEPS;        // steps: tile u / STEPS, part u % STEPS
+  int u0, u1;                                                  // steps: tile u / STEPS, part u % STEPS
+  {
+    const int t0 = cp[n], len = cp[n + 1] - t0;                // this workgroup's share of the column's list
+    u0 = (t0 + (int)((int64_t)len * chunk / prm.split)) * STEPS;
+    u1 = (t0 + (int)((int64_t)len * (chunk + 1) / prm.split)) * STEPS;
+  }
   const unsigned lds_addr = (unsigned)(uintptr_t)(lds_ptr_t)lds;
 
   const unsigned short* qg = (const unsigned short*)prm.q + b * prm.qs[0] + h * prm.qs[1];
@@ -438,6 +464,20 @@ __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
       }
   }
 
+  if (prm.split > 1) {   // unscaled fp32 parts; sum_parts_kernel adds them up
+    const int64_t poff = ((int64_t)chunk * prm.B * prm.H + bh) * prm.N * D;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const int64_t off = krow * D + 32 * db + 8 * i4 + 4 * g;
+        store_out4<BF16>(prm.part_dk + poff, off, true, dkacc[db][4 * i4], dkacc[db][4 * i4 + 1], dkacc[db][4 * i4 + 2],
+                         dkacc[db][4 * i4 + 3]);
+        store_out4<BF16>(prm.part_dv + poff, off, true, dvacc[db][4 * i4], dvacc[db][4 * i4 + 1], dvacc[db][4 * i4 + 2],
+                         dvacc[db][4 * i4 + 3]);
+      }
+    return;
+  }
   const int64_t hoff = (int64_t)bh * prm.N * D;
   void* kbase = prm.out_f32 ? (void*)((float*)prm.dk + hoff) : (void*)((unsigned short*)prm.dk + hoff);
   void* vbase = prm.out_f32 ? (void*)((float*)prm.dv + hoff) : (void*)((unsigned short*)prm.dv + hoff);
@@ -454,11 +494,38 @@ __global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
 }
 
 // ---------------------------------------------------------------------------------------
+// split > 1: out = scale * sum of the fp32 parts, rounded to the result type.  blockIdx.y: 0 dQ, 1 dK, 2 dV.
+// ---------------------------------------------------------------------------------------
+template <bool BF16>
+__global__ __launch_bounds__(256) void sum_parts_kernel(const BwdParams prm, int64_t quads) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;     // one thread per 4 consecutive values
+  if (i >= quads) return;
+  const float* part = blockIdx.y == 0 ? prm.part_dq : (blockIdx.y == 1 ? prm.part_dk : prm.part_dv);
+  void* out = blockIdx.y == 0 ? prm.dq : (blockIdx.y == 1 ? prm.dk : prm.dv);
+  const float scale = blockIdx.y == 2 ? 1.0f : prm.sm_scale;
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int c = 0; c < prm.split; ++c) acc += reinterpret_cast<const floatx4*>(part)[c * quads + i];
+  store_out4<BF16>(out, 4 * i, prm.out_f32, acc[0] * scale, acc[1] * scale, acc[2] * scale, acc[3] * scale);
+}
+
+// ---------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------
+// Workgroups per row / column list.  One is enough when the launch has at least four workgroups
+// per compute unit; a single long head would otherwise walk its lists on a fraction of the GPU.
+static int bwd_split(int B, int H, int N) {
+  const int64_t lists = (int64_t)B * H * (N / 64), want = 4 * (int64_t)compute_units();
+  if (lists >= want) return 1;
+  int64_t s = (want + lists - 1) / lists;
+  const int cap = N / 64 / 8 > 1 ? N / 64 / 8 : 1;        // a share should have a few tiles even in a dense list
+  if (s > cap) s = cap;
+  return (int)(s > 8 ? 8 : s);
+}
+
 size_t bwd_workspace_bytes(int B, int H, int N, int D) {
-  (void)D;
-  return (size_t)B * H * N * sizeof(float);   // delta
+  const size_t delta = (size_t)B * H * N * sizeof(float);
+  const int split = bwd_split(B, H, N);
+  return delta + (split > 1 ? (size_t)3 * split * B * H * N * D * sizeof(float) : 0);   // + parts of dQ, dK, dV
 }
 
 template <int D, bool BF16, bool EW, bool PB>
@@ -480,9 +547,13 @@ static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
   const int BH = prm.B * prm.H;
   constexpr int RPB = 256 / (D / 8);
   hipLaunchKernelGGL((delta_kernel<D, BF16>), dim3((prm.N + RPB - 1) / RPB, BH), dim3(256), 0, st, prm);
-  const int grid = ((BH + 7) / 8) * 8 * prm.nb;   // heads in groups of 8, the last group padded
+  const int grid = ((BH + 7) / 8) * 8 * prm.nb * prm.split;   // heads in groups of 8, the last group padded
   hipLaunchKernelGGL((dq_kernel<D, BF16, EW, PB, KB>), dim3(grid), dim3(128), CQ::LDS_BYTES, st, prm);
   hipLaunchKernelGGL((dkdv_kernel<D, BF16, EW, PB, QB>), dim3(grid), dim3(128), CK::LDS_BYTES, st, prm);
+  if (prm.split > 1) {
+    const int64_t quads = (int64_t)BH * prm.N * D / 4;
+    hipLaunchKernelGGL((sum_parts_kernel<BF16>), dim3((unsigned)((quads + 255) / 256), 3), dim3(256), 0, st, prm, quads);
+  }
 }
 
 int launch_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
@@ -497,6 +568,13 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* o, const
   prm.bits_rows = (const unsigned long long*)bits_rows; prm.bits_cols = (const unsigned long long*)bits_cols;
   prm.B = s.B; prm.H = s.H; prm.N = s.N; prm.nb = s.N / 64; prm.Bm = s.Bm; prm.Hm = s.Hm;
   prm.out_f32 = s.out_dtype == BSATTN_F32;
+  prm.split = bwd_split(s.B, s.H, s.N);
+  {
+    const size_t one = (size_t)prm.split * s.B * s.H * s.N * s.D;
+    prm.part_dq = (float*)ws + (size_t)s.B * s.H * s.N;
+    prm.part_dk = prm.part_dq + one;
+    prm.part_dv = prm.part_dk + one;
+  }
   prm.sm_scale = s.sm_scale;
   prm.qk_scale = s.sm_scale * kLog2e;
   for (int i = 0; i < 3; ++i) {

@@ -797,7 +797,7 @@ static unsigned long long next_epoch() {
   return e;
 }
 
-static int compute_units() {
+int compute_units() {
   int dev = 0, cus = 256;
   if (hipGetDevice(&dev) == hipSuccess) {
     int v = 0;

@@ -29,6 +29,7 @@ struct AttnShape {
 };
 
 // attn_fwd.hip
+int compute_units();   // of the current device (256 if the query fails)
 size_t fwd_workspace_bytes(int B, int H, int N, int D);
 int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                const int32_t* row_ptr, const int32_t* col_idx, const uint8_t* tile_partial,
