@@ -157,6 +157,10 @@ int bsattn_fwd_elementwise(const void* q, const void* k, const void* v, void* o,
  * The gradient algebra is the reference's (fa2_bwd.py:17,57-74,117-130,232,284) evaluated
  * over exactly the kept tiles.
  * ---------------------------------------------------------------------------------- */
+
+/* Bytes of workspace bsattn_bwd needs: delta = rowsum(O * dO), and for launches with few row
+ * blocks the fp32 parts of dQ, dK, dV of row / column lists walked by several workgroups.
+ * Depends on the shape and on the number of compute units of the current device. */
 int bsattn_bwd_workspace(int B, int H, int N, int D, size_t* bytes);
 
 /* q,k,v,o,d_o: [B,H,N,D] fp16/bf16 with their own strides; lse from bsattn_fwd.
