@@ -49,6 +49,25 @@ def test_c4_n32000_block_causal(dev, keep):
     assert same_up_to_rounding(o2[0, 0, :-64], o[0, 0, :-64])
 
 
+def test_very_long_sequence_n262144(dev):
+    """4096 row blocks: the row-pointer searches leave their one-load-per-lane form (binary search),
+    and a range's column list no longer fits its LDS staging area.  Sparse mask (a band, a few random
+    tiles and one long row block); forward on sampled row blocks, lists bit-exact."""
+    import fa2_custom_mask as fm
+    N, nb = 262144, 4096
+    g = torch.Generator().manual_seed(1240)
+    idx = torch.arange(nb)
+    mask = ((idx[:, None] - idx[None, :]).abs() <= 2) | (torch.rand(nb, nb, generator=g) < 0.001)
+    mask[2000, ::2] = True                       # 2048 + kept tiles in one row block
+    mask[2001, :] = False                        # a row block without any
+    mask = mask.reshape(1, 1, nb, nb)
+    groups, n_list = fm.build_groups_from_block_mask(mask.to(dev))
+    g_ref, n_ref = orc.build_groups_from_block_mask(mask.numpy())
+    assert np.array_equal(groups.cpu().numpy(), g_ref) and np.array_equal(n_list.cpu().numpy(), n_ref)
+    q, k, v, o = sampled_forward_check(dev, N, 64, mask, 1240, [0, 1, 1999, 2000, 2002, 4095])
+    assert float(np.abs(o[0, 0, 2001 * 64:2002 * 64]).max()) == 0.0
+
+
 def test_c2_dense_elementwise_mask_n6400(dev):
     """C2: preprocessing from a dense N x N bool mask (tile-constant) feeds the same result."""
     import fa2_custom_mask as fm
