@@ -326,7 +326,7 @@ __global__ __launch_bounds__(128, 2) void dq_kernel(const BwdParams prm) {
 // QB: 32-query blocks of a tile handled per step (2: a whole tile; 1: a tile in two halves, which
 // halves the fragments in flight).
 template <int D, bool BF16, bool EW, bool PB, int QB>
-__global__ __launch_bounds__(128) void dkdv_kernel(const BwdParams prm) {
+__global__ __launch_bounds__(128, QB == 1 ? 2 : 1) void dkdv_kernel(const BwdParams prm) {
   using C = BwdCfg<D, EW, 32 * QB>;
   constexpr int KS = D / 16, DB = D / 32, STEPS = 2 / QB;
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
@@ -531,10 +531,12 @@ size_t bwd_workspace_bytes(int B, int H, int N, int D) {
 template <int D, bool BF16, bool EW, bool PB>
 static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
   using C = BwdCfg<D, EW>;
-  constexpr int KB = D == 128 ? 1 : 2;          // dq_kernel walks D = 128 tiles in two halves
+  constexpr int KB = D == 128 ? 1 : 2;          // dq_kernel walks D = 128 tiles in two halves (no gain at D = 64: two wavefronts per SIMD anyway)
   using CQ = BwdCfg<D, EW, 32 * KB>;
-  constexpr int QB = 2;   // dkdv_kernel keeps one wavefront per SIMD either way (K, V, dK, dV of 32 keys are 192
-                          // registers at D = 128); halves were measured slower there (718 against 688 us, C5)
+  // dkdv_kernel: halves at D = 64 (191 instead of 318 registers: two wavefronts per SIMD; B*H = 32 N = 8192 dense
+  // block-causal backward 1417 -> 1167 us).  At D = 128 it keeps one wavefront per SIMD either way (K, V, dK, dV of
+  // 32 keys are 192 registers) and halves were measured slower (718 against 688 us, C5).
+  constexpr int QB = D == 64 ? 1 : 2;
   using CK = BwdCfg<D, EW, 32 * QB>;
   static bool configured = false;   // raising the dynamic LDS limit is idempotent
   if (!configured) {
