@@ -15,7 +15,7 @@ const char* bsattn_strerror(int code) {
     case BSATTN_ERR_NULL: return "a required pointer is NULL";
     case BSATTN_ERR_SHAPE: return "bad shape: sizes must be positive, N a multiple of 64, mask batch/head sizes 1 or equal to B/H";
     case BSATTN_ERR_DTYPE: return "unsupported dtype code";
-    case BSATTN_ERR_HEAD_DIM: return "head dimension must be 64 or 128";
+    case BSATTN_ERR_HEAD_DIM: return "head dimension must be 64, 128 or 256";
     case BSATTN_ERR_STRIDE: return "innermost stride must be 1 and rows 16-byte aligned";
     case BSATTN_ERR_WORKSPACE: return "workspace missing or too small";
     case BSATTN_ERR_LAUNCH: return "HIP launch failed";
@@ -78,7 +78,7 @@ int bsattn_tail_mask_tiles(int Bm, int Hm, int nb, int valid_last, int transpose
 static int check_attn(int Bm, int Hm, int B, int H, int N, int D, int dtype, int out_dtype) {
   if (B <= 0 || H <= 0 || N <= 0 || N % BSATTN_TILE != 0) return BSATTN_ERR_SHAPE;
   if (!((Bm == 1 || Bm == B) && (Hm == 1 || Hm == H))) return BSATTN_ERR_SHAPE;
-  if (D != 64 && D != 128) return BSATTN_ERR_HEAD_DIM;
+  if (D != 64 && D != 128 && D != 256) return BSATTN_ERR_HEAD_DIM;
   if (dtype != BSATTN_F16 && dtype != BSATTN_BF16) return BSATTN_ERR_DTYPE;
   if (out_dtype != dtype && out_dtype != BSATTN_F32) return BSATTN_ERR_DTYPE;
   if ((int64_t)B * H > 65535) return BSATTN_ERR_RANGE;

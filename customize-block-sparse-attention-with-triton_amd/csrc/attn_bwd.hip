@@ -17,6 +17,7 @@
 // double buffer (one barrier per tile).
 #include "common.h"
 #include "kernel_util.h"
+#include <type_traits>
 
 namespace bsattn {
 
@@ -177,9 +178,10 @@ __device__ __forceinline__ void head_and_block(int L, int BH, int nb, int& bh, i
 // tile is walked in two steps of 32 keys; the staged halves are 8 KB, four workgroups fit a compute
 // unit and the wavefront stays within 256 registers: two wavefronts per SIMD.
 template <int D, bool BF16, bool EW, bool PB, int KB>
-__global__ __launch_bounds__(128, 2) void dq_kernel(const BwdParams prm) {
+__global__ __launch_bounds__(128, D == 256 ? 1 : 2) void dq_kernel(const BwdParams prm) {
   using C = BwdCfg<D, EW, 32 * KB>;
   constexpr int KS = D / 16, DB = D / 32, STEPS = 2 / KB;
+  constexpr int PORTIONS = D == 256 ? 2 : 1, KSP = KS / PORTIONS;   // D = 256: the fragments of the first products in two portions
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int ln = lane & 31, g = lane >> 5;
@@ -247,26 +249,29 @@ __global__ __launch_bounds__(128, 2) void dq_kernel(const BwdParams prm) {
 
     // All operand fragments of a block of MFMAs are read from LDS before the block starts: a read
     // issued next to the MFMA that consumes it costs a full LDS latency per MFMA.
-    uintx4 fk[KB][KS], fv[KB][KS];
-#pragma unroll
-    for (int s = 0; s < KS; ++s)
-#pragma unroll
-      for (int kb = 0; kb < KB; ++kb) {
-        fk[kb][s] = frag_rows<D>(kt, 32 * kb, s, ln, g);
-        fv[kb][s] = frag_rows<D>(vt, 32 * kb, s, ln, g);
-      }
-    __builtin_amdgcn_sched_barrier(0);
     floatx16 sacc[KB], dpacc[KB];
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb) { sacc[kb] = zero16(); dpacc[kb] = zero16(); }
 #pragma unroll
-    for (int s = 0; s < KS; ++s)
+    for (int pt = 0; pt < PORTIONS; ++pt) {
+      uintx4 fk[KB][KSP], fv[KB][KSP];
 #pragma unroll
-      for (int kb = 0; kb < KB; ++kb) {
-        sacc[kb] = mfma_qk<BF16>(fk[kb][s], qfr[s], sacc[kb]);      // S^T = K Q^T
-        dpacc[kb] = mfma_qk<BF16>(fv[kb][s], dofr[s], dpacc[kb]);   // dP^T = V dO^T
-      }
-    __builtin_amdgcn_sched_barrier(0);
+      for (int s = 0; s < KSP; ++s)
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+          fk[kb][s] = frag_rows<D>(kt, 32 * kb, pt * KSP + s, ln, g);
+          fv[kb][s] = frag_rows<D>(vt, 32 * kb, pt * KSP + s, ln, g);
+        }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < KSP; ++s)
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+          sacc[kb] = mfma_qk<BF16>(fk[kb][s], qfr[pt * KSP + s], sacc[kb]);      // S^T = K Q^T
+          dpacc[kb] = mfma_qk<BF16>(fv[kb][s], dofr[pt * KSP + s], dpacc[kb]);   // dP^T = V dO^T
+        }
+      __builtin_amdgcn_sched_barrier(0);
+    }
     if constexpr (EW) {
       unsigned long long mw = *reinterpret_cast<const unsigned long long*>(
           vt + C::TILE_BYTES + C::STAT_BYTES + (32 * wv + ln) * 8);
@@ -325,10 +330,15 @@ __global__ __launch_bounds__(128, 2) void dq_kernel(const BwdParams prm) {
 // ---------------------------------------------------------------------------------------
 // QB: 32-query blocks of a tile handled per step (2: a whole tile; 1: a tile in two halves, which
 // halves the fragments in flight).
-template <int D, bool BF16, bool EW, bool PB, int QB>
-__global__ __launch_bounds__(128, QB == 1 ? 2 : 1) void dkdv_kernel(const BwdParams prm) {
+// DH: -1, or at D = 256 the half (0 / 1) of the head dimension whose dK and dV columns this launch
+// accumulates and writes (the first products always contract over the whole head dimension): with
+// 128 columns at a time the accumulators and K, V of 32 keys are 256 registers instead of 384.
+template <int D, bool BF16, bool EW, bool PB, int QB, int DH>
+__global__ __launch_bounds__(128, (QB == 1 && D == 64) ? 2 : 1) void dkdv_kernel(const BwdParams prm) {
   using C = BwdCfg<D, EW, 32 * QB>;
-  constexpr int KS = D / 16, DB = D / 32, STEPS = 2 / QB;
+  constexpr int KS = D / 16, STEPS = 2 / QB;
+  constexpr int DB = DH < 0 ? D / 32 : D / 64, DB0 = DH < 0 ? 0 : DH * DB;   // 32-column blocks of this launch, the first one
+  constexpr int PORTIONS = D == 256 ? 2 : 1, KSP = KS / PORTIONS;            // fragments of the first products in portions
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int ln = lane & 31, g = lane >> 5;
@@ -396,26 +406,29 @@ __global__ __launch_bounds__(128, QB == 1 ? 2 : 1) void dkdv_kernel(const BwdPar
     const float* st_dlt = st_lse + 64;
 
     // operand fragments are read from LDS ahead of the block of MFMAs that consumes them
-    uintx4 fq[QB][KS], fg[QB][KS];
-#pragma unroll
-    for (int s = 0; s < KS; ++s)
-#pragma unroll
-      for (int qb = 0; qb < QB; ++qb) {
-        fq[qb][s] = frag_rows<D>(qt, 32 * qb, s, ln, g);
-        fg[qb][s] = frag_rows<D>(gt, 32 * qb, s, ln, g);
-      }
-    __builtin_amdgcn_sched_barrier(0);
     floatx16 sacc[QB], dpacc[QB];
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) { sacc[qb] = zero16(); dpacc[qb] = zero16(); }
 #pragma unroll
-    for (int s = 0; s < KS; ++s)
+    for (int pt = 0; pt < PORTIONS; ++pt) {
+      uintx4 fq[QB][KSP], fg[QB][KSP];
 #pragma unroll
-      for (int qb = 0; qb < QB; ++qb) {
-        sacc[qb] = mfma_qk<BF16>(fq[qb][s], kfr[s], sacc[qb]);      // S = Q K^T
-        dpacc[qb] = mfma_qk<BF16>(fg[qb][s], vfr[s], dpacc[qb]);    // dP = dO V^T
-      }
-    __builtin_amdgcn_sched_barrier(0);
+      for (int s = 0; s < KSP; ++s)
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) {
+          fq[qb][s] = frag_rows<D>(qt, 32 * qb, pt * KSP + s, ln, g);
+          fg[qb][s] = frag_rows<D>(gt, 32 * qb, pt * KSP + s, ln, g);
+        }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int s = 0; s < KSP; ++s)
+#pragma unroll
+        for (int qb = 0; qb < QB; ++qb) {
+          sacc[qb] = mfma_qk<BF16>(fq[qb][s], kfr[pt * KSP + s], sacc[qb]);      // S = Q K^T
+          dpacc[qb] = mfma_qk<BF16>(fg[qb][s], vfr[pt * KSP + s], dpacc[qb]);    // dP = dO V^T
+        }
+      __builtin_amdgcn_sched_barrier(0);
+    }
     if constexpr (EW) {
       unsigned long long mw = *reinterpret_cast<const unsigned long long*>(
           gt + C::TILE_BYTES + C::STAT_BYTES + (32 * wv + ln) * 8);
@@ -430,8 +443,8 @@ __global__ __launch_bounds__(128, QB == 1 ? 2 : 1) void dkdv_kernel(const BwdPar
     for (int ts = 0; ts < 2 * QB; ++ts)
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        fgt[ts][db] = frag_cols<D, BF16 && !PB>(gt, db, ts, lane);
-        fqt[ts][db] = frag_cols<D, BF16 && !PB>(qt, db, ts, lane);
+        fgt[ts][db] = frag_cols<D, BF16 && !PB>(gt, DB0 + db, ts, lane);
+        fqt[ts][db] = frag_cols<D, BF16 && !PB>(qt, DB0 + db, ts, lane);
       }
     __builtin_amdgcn_sched_barrier(0);
     // rows of the results are queries: register i of block qb <-> query 32qb + 8(i/4) + 4g + i%4
@@ -470,7 +483,7 @@ __global__ __launch_bounds__(128, QB == 1 ? 2 : 1) void dkdv_kernel(const BwdPar
     for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
-        const int64_t off = krow * D + 32 * db + 8 * i4 + 4 * g;
+        const int64_t off = krow * D + 32 * (DB0 + db) + 8 * i4 + 4 * g;
         store_out4<BF16>(prm.part_dk + poff, off, true, dkacc[db][4 * i4], dkacc[db][4 * i4 + 1], dkacc[db][4 * i4 + 2],
                          dkacc[db][4 * i4 + 3]);
         store_out4<BF16>(prm.part_dv + poff, off, true, dvacc[db][4 * i4], dvacc[db][4 * i4 + 1], dvacc[db][4 * i4 + 2],
@@ -485,7 +498,7 @@ __global__ __launch_bounds__(128, QB == 1 ? 2 : 1) void dkdv_kernel(const BwdPar
   for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int i4 = 0; i4 < 4; ++i4) {
-      const int64_t off = krow * D + 32 * db + 8 * i4 + 4 * g;
+      const int64_t off = krow * D + 32 * (DB0 + db) + 8 * i4 + 4 * g;
       store_out4<BF16>(kbase, off, prm.out_f32, dkacc[db][4 * i4] * prm.sm_scale, dkacc[db][4 * i4 + 1] * prm.sm_scale,
                        dkacc[db][4 * i4 + 2] * prm.sm_scale, dkacc[db][4 * i4 + 3] * prm.sm_scale);
       store_out4<BF16>(vbase, off, prm.out_f32, dvacc[db][4 * i4], dvacc[db][4 * i4 + 1], dvacc[db][4 * i4 + 2],
@@ -531,19 +544,26 @@ size_t bwd_workspace_bytes(int B, int H, int N, int D) {
 template <int D, bool BF16, bool EW, bool PB>
 static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
   using C = BwdCfg<D, EW>;
-  constexpr int KB = D == 128 ? 1 : 2;          // dq_kernel walks D = 128 tiles in two halves (no gain at D = 64: two wavefronts per SIMD anyway)
+  constexpr int KB = D >= 128 ? 1 : 2;          // dq_kernel walks D >= 128 tiles in two halves (no gain at D = 64: two wavefronts per SIMD anyway)
   using CQ = BwdCfg<D, EW, 32 * KB>;
   // dkdv_kernel: halves at D = 64 (191 instead of 318 registers: two wavefronts per SIMD; B*H = 32 N = 8192 dense
   // block-causal backward 1417 -> 1167 us).  At D = 128 it keeps one wavefront per SIMD either way (K, V, dK, dV of
   // 32 keys are 192 registers) and halves were measured slower (718 against 688 us, C5).
-  constexpr int QB = D == 64 ? 1 : 2;
+  constexpr int QB = D == 128 ? 2 : 1;   // (D = 256: halves, and the head dimension of dK, dV in two launches)
   using CK = BwdCfg<D, EW, 32 * QB>;
   static bool configured = false;   // raising the dynamic LDS limit is idempotent
   if (!configured) {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dq_kernel<D, BF16, EW, PB, KB>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, CQ::LDS_BYTES);
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv_kernel<D, BF16, EW, PB, QB>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, CK::LDS_BYTES);
+    if constexpr (D == 256) {
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv_kernel<D, BF16, EW, PB, QB, 0>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, CK::LDS_BYTES);
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv_kernel<D, BF16, EW, PB, QB, 1>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, CK::LDS_BYTES);
+    } else {
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv_kernel<D, BF16, EW, PB, QB, -1>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, CK::LDS_BYTES);
+    }
     configured = true;
   }
   const int BH = prm.B * prm.H;
@@ -551,7 +571,12 @@ static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
   hipLaunchKernelGGL((delta_kernel<D, BF16>), dim3((prm.N + RPB - 1) / RPB, BH), dim3(256), 0, st, prm);
   const int grid = ((BH + 7) / 8) * 8 * prm.nb * prm.split;   // heads in groups of 8, the last group padded
   hipLaunchKernelGGL((dq_kernel<D, BF16, EW, PB, KB>), dim3(grid), dim3(128), CQ::LDS_BYTES, st, prm);
-  hipLaunchKernelGGL((dkdv_kernel<D, BF16, EW, PB, QB>), dim3(grid), dim3(128), CK::LDS_BYTES, st, prm);
+  if constexpr (D == 256) {   // the two halves of the head dimension of dK, dV in two launches
+    hipLaunchKernelGGL((dkdv_kernel<D, BF16, EW, PB, QB, 0>), dim3(grid), dim3(128), CK::LDS_BYTES, st, prm);
+    hipLaunchKernelGGL((dkdv_kernel<D, BF16, EW, PB, QB, 1>), dim3(grid), dim3(128), CK::LDS_BYTES, st, prm);
+  } else {
+    hipLaunchKernelGGL((dkdv_kernel<D, BF16, EW, PB, QB, -1>), dim3(grid), dim3(128), CK::LDS_BYTES, st, prm);
+  }
   if (prm.split > 1) {
     const int64_t quads = (int64_t)BH * prm.N * D / 4;
     hipLaunchKernelGGL((sum_parts_kernel<BF16>), dim3((unsigned)((quads + 255) / 256), 3), dim3(256), 0, st, prm, quads);
@@ -587,21 +612,22 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* o, const
   // reference's forward does with P, fa2_fwd.py:189) and no tile needs converting; fp32 gradients of
   // bf16 inputs keep P and dS in fp16.
   const bool pb = bf && !prm.out_f32;
-  if (bits_rows == nullptr) {
-    if (s.D == 64 && !bf) launch_bwd_t<64, false, false, false>(prm, st);
-    else if (s.D == 64 && pb) launch_bwd_t<64, true, false, true>(prm, st);
-    else if (s.D == 64) launch_bwd_t<64, true, false, false>(prm, st);
-    else if (s.D == 128 && !bf) launch_bwd_t<128, false, false, false>(prm, st);
-    else if (pb) launch_bwd_t<128, true, false, true>(prm, st);
-    else launch_bwd_t<128, true, false, false>(prm, st);
-  } else {   // elementwise mask
-    if (s.D == 64 && !bf) launch_bwd_t<64, false, true, false>(prm, st);
-    else if (s.D == 64 && pb) launch_bwd_t<64, true, true, true>(prm, st);
-    else if (s.D == 64) launch_bwd_t<64, true, true, false>(prm, st);
-    else if (s.D == 128 && !bf) launch_bwd_t<128, false, true, false>(prm, st);
-    else if (pb) launch_bwd_t<128, true, true, true>(prm, st);
-    else launch_bwd_t<128, true, true, false>(prm, st);
-  }
+  const bool ew = bits_rows != nullptr;
+  auto pick = [&](auto dc) {
+    constexpr int DD = decltype(dc)::value;
+    if (!ew) {
+      if (!bf) launch_bwd_t<DD, false, false, false>(prm, st);
+      else if (pb) launch_bwd_t<DD, true, false, true>(prm, st);
+      else launch_bwd_t<DD, true, false, false>(prm, st);
+    } else {   // elementwise mask
+      if (!bf) launch_bwd_t<DD, false, true, false>(prm, st);
+      else if (pb) launch_bwd_t<DD, true, true, true>(prm, st);
+      else launch_bwd_t<DD, true, true, false>(prm, st);
+    }
+  };
+  if (s.D == 64) pick(std::integral_constant<int, 64>{});
+  else if (s.D == 128) pick(std::integral_constant<int, 128>{});
+  else pick(std::integral_constant<int, 256>{});
   return launch_status();
 }
 

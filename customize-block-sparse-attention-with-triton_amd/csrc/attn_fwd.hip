@@ -822,12 +822,13 @@ static size_t slots_bytes(int B, int H, int W, int D) {
 }
 
 size_t fwd_workspace_bytes(int B, int H, int N, int D) {
+  if (D == 256) return 256;     // one wavefront pair per row block: nothing is shared between workgroups
   const int nb = N / 64;
   const int W = groups_per_head(B, H, nb, D);
   return slots_bytes(B, H, W, D) + (size_t)B * H * W * sizeof(unsigned long long);
 }
 
-void launch_fwd_pair(const FwdParams& prm, int dt, bool elementwise, hipStream_t st);   // attn_fwd_pair.hip
+void launch_fwd_pair(const FwdParams& prm, int D, int dt, bool elementwise, hipStream_t st);   // attn_fwd_pair.hip
 // D = 128 with enough row blocks in the launch to fill the chip goes to the kernel that gives each
 // row block to one wavefront pair (two wavefronts per SIMD, no merges between workgroups).  With
 // fewer row blocks its critical path is the longest row, which the host cannot see (the lists
@@ -879,8 +880,8 @@ int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
   for (int i = 0; i < 3; ++i) { prm.qs[i] = s.qs[i]; prm.ks[i] = s.ks[i]; prm.vs[i] = s.vs[i]; prm.os[i] = s.os[i]; }
   const bool bf = s.dtype == BSATTN_BF16;
   const int BH = s.B * s.H;
-  if (s.D == 128 && use_pair_kernel((int64_t)BH * prm.nb, prm.nb)) {
-    launch_fwd_pair(prm, !bf ? 0 : (prm.out_f32 ? 1 : 2), tile_bits != nullptr, st);
+  if (s.D == 256 || (s.D == 128 && use_pair_kernel((int64_t)BH * prm.nb, prm.nb))) {   // (D = 256 has no other kernel)
+    launch_fwd_pair(prm, s.D, !bf ? 0 : (prm.out_f32 ? 1 : 2), tile_bits != nullptr, st);
     return launch_status();
   }
   // bf16 with a bf16-typed result: P is rounded to bf16 as well (the reference rounds P to the type of

@@ -1,4 +1,6 @@
-// Block-sparse FlashAttention-2 forward, head dimension 128, for launches with many row blocks.
+// Block-sparse FlashAttention-2 forward, head dimension 128 for launches with many row blocks, and
+// head dimension 256 (the only forward kernel for it; one wavefront per SIMD there, K and V fragments
+// taken from LDS in two portions).
 //
 // At D = 128 a wavefront that owns 64 queries needs all 512 registers of its SIMD, so the
 // general kernel (attn_fwd.hip) runs one wavefront per SIMD and is bound by instruction issue.
@@ -19,11 +21,13 @@
 namespace bsattn {
 
 constexpr int PAIR_COLS_CAP = 1024;                               // column indices of the row block kept in LDS
-constexpr int PAIR_LDS_BYTES = 2 * 16384 + 512 + PAIR_COLS_CAP * 4;   // K tile, V tile, mask words, columns
+template <int D> constexpr int pair_lds_bytes() { return 2 * 64 * 2 * D + 512 + PAIR_COLS_CAP * 4; }   // K tile, V tile, mask words, columns
 
-template <int DT, bool EW>
-__global__ __launch_bounds__(128, 2) void fwd_pair_kernel(const FwdParams prm) {
-  constexpr int D = 128, KS = D / 16, DB = D / 32, CPR = D / 8, ROWB = 2 * D, TILE_BYTES = 64 * ROWB;
+template <int D, int DT, bool EW>
+__global__ __launch_bounds__(128, D == 128 ? 2 : 1) void fwd_pair_kernel(const FwdParams prm) {
+  constexpr int KS = D / 16, DB = D / 32, CPR = D / 8, ROWB = 2 * D, TILE_BYTES = 64 * ROWB;
+  constexpr int PORTIONS = D / 128;              // K and V fragments are read in this many portions
+  constexpr int KSP = KS / PORTIONS, DBP = DB / PORTIONS;
   constexpr bool BF16 = DT != 0;
   constexpr bool PB = DT == 2;                   // P rounded to bf16, second product in bf16 (V as it is)
   constexpr bool FOLD = !BF16;
@@ -91,14 +95,17 @@ __global__ __launch_bounds__(128, 2) void fwd_pair_kernel(const FwdParams prm) {
 
   // asynchronous tile copies: copy instruction j covers tile rows [4j, 4j+4); this wavefront issues
   // the instructions [HALF w, HALF (w+1)) of every tile (and 256 of the 512 bytes of mask words)
-  constexpr int RPI = 64 / CPR, KPER = 4;
-  unsigned koff[KPER], voff;
+  // (the swizzles repeat every 16 rows for K and every 4 rows for V: KPER / VPER instructions)
+  constexpr int RPI = 64 / CPR, KPER = 16 / RPI, VPER = RPI >= 4 ? 1 : 4 / RPI;
+  unsigned koff[KPER], voff[VPER];
   {
     const int row0 = lane / CPR, ch = lane % CPR;
 #pragma unroll
     for (int par = 0; par < KPER; ++par)
       koff[par] = 2u * (unsigned)(row0 * (int)prm.ks[2] + ((ch ^ k_swz<D>(par * RPI + row0)) * 8));
-    voff = 2u * (unsigned)(row0 * (int)prm.vs[2] + ((ch ^ v_swz<D>(row0)) * 8));
+#pragma unroll
+    for (int par = 0; par < VPER; ++par)
+      voff[par] = 2u * (unsigned)(row0 * (int)prm.vs[2] + ((ch ^ v_swz<D>(par * RPI + row0)) * 8));
   }
   auto k_copy = [&](int cb, int t) {
     const unsigned short* tile = kg + (int64_t)cb * 64 * prm.ks[2];
@@ -118,10 +125,10 @@ __global__ __launch_bounds__(128, 2) void fwd_pair_kernel(const FwdParams prm) {
 #pragma unroll
     for (int jj = 0; jj < HALF; ++jj) {
       const int j = w * HALF + jj;
-      tile_load_async_one(tile + (int64_t)j * RPI * prm.vs[2], voff, lds_v_addr + j * 1024);
+      tile_load_async_one(tile + (int64_t)j * RPI * prm.vs[2], voff[jj % VPER], lds_v_addr + j * 1024);
     }
   };
-  static_assert(HALF % KPER == 0, "the K swizzle pattern of a wavefront's instructions starts at phase 0");
+  static_assert(HALF % KPER == 0 && HALF % VPER == 0, "the swizzle patterns of a wavefront's instructions start at phase 0");
 
   // fragment addresses (as in attn_fwd.hip)
   int kaddr[2][KS];
@@ -171,25 +178,29 @@ __global__ __launch_bounds__(128, 2) void fwd_pair_kernel(const FwdParams prm) {
     const bool has1 = t + 1 < t1;
     const int cxn = has1 ? __builtin_amdgcn_readfirstlane(col_of(t + 1)) : 0;
     const bool partial = EW && (cx >> 30) != 0;
-    // ---- K fragments (and the mask word of this lane's query) ----
-    uintx4 kfr[2][KS];
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int s = 0; s < KS; ++s) kfr[kb][s] = *reinterpret_cast<const uintx4*>(lds_k + kaddr[kb][s]);
-    unsigned long long mw = 0ull;
-    if constexpr (EW) { if (partial) mw = lds_bits[32 * w + ln] >> (4 * g); }
-    lds_wait();
-    __syncthreads();                                // both wavefronts hold their K fragments: the K buffer is free
-    if (has1) k_copy(cxn & COL_MASK, t + 1);
-    // ---- S^T = K Q^T (- m when FOLD) ----
+    // ---- S^T = K Q^T (- m when FOLD); the K fragments (and the mask word of this lane's query) ----
     floatx16 s0, s1;
 #pragma unroll
     for (int i = 0; i < 16; ++i) { s0[i] = 0.f; s1[i] = 0.f; }
+    unsigned long long mw = 0ull;
 #pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      s0 = mfma_qk<BF16>(kfr[0][s], qf[0][s], s0);
-      s1 = mfma_qk<BF16>(kfr[1][s], qf[0][s], s1);
+    for (int pt = 0; pt < PORTIONS; ++pt) {
+      uintx4 kfr[2][KSP];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int s = 0; s < KSP; ++s) kfr[kb][s] = *reinterpret_cast<const uintx4*>(lds_k + kaddr[kb][pt * KSP + s]);
+      if (pt == PORTIONS - 1) {
+        if constexpr (EW) { if (partial) mw = lds_bits[32 * w + ln] >> (4 * g); }
+        lds_wait();
+        __syncthreads();                            // both wavefronts hold their K fragments: the K buffer is free
+        if (has1) k_copy(cxn & COL_MASK, t + 1);
+      }
+#pragma unroll
+      for (int s = 0; s < KSP; ++s) {
+        s0 = mfma_qk<BF16>(kfr[0][s], qf[0][pt * KSP + s], s0);
+        s1 = mfma_qk<BF16>(kfr[1][s], qf[0][pt * KSP + s], s1);
+      }
     }
     if constexpr (FOLD) {
       s0 = mfma_qk<BF16>(ones_frag, mfrag, s0);
@@ -218,33 +229,38 @@ __global__ __launch_bounds__(128, 2) void fwd_pair_kernel(const FwdParams prm) {
     // ---- V^T fragments ----
     if (has1) wait_vm<KOPS>(); else wait_vm<0>();   // this wavefront's half of V(t) has landed (K(t+1) may be in flight)
     if (t > t0) __syncthreads();                    // ... and the other half (the first tile was waited for above)
-    uintx4 vfr[4][DB];
+    // ---- O^T += V^T P^T, the V^T fragments taken in PORTIONS portions ----
 #pragma unroll
-    for (int ts = 0; ts < 4; ++ts)
+    for (int pt = 0; pt < PORTIONS; ++pt) {
+      uintx4 vfr[4][DBP];
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        uintx4 a;
+      for (int ts = 0; ts < 4; ++ts)
 #pragma unroll
-        for (int jh = 0; jh < 2; ++jh) {
-          const int key = 16 * ts + 8 * jh + vkey0, col = 32 * db + vcol0;
-          const int addr = key * ROWB + (((col >> 3) ^ v_swz<D>(key)) * 16) + (col & 7) * 2;
-          const short4v rr = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (short4v __attribute__((address_space(3)))*)(lds_v + addr));
-          const uintx2 r2 = __builtin_bit_cast(uintx2, rr);
-          a[2 * jh] = r2[0]; a[2 * jh + 1] = r2[1];
+        for (int db = 0; db < DBP; ++db) {
+          uintx4 a;
+#pragma unroll
+          for (int jh = 0; jh < 2; ++jh) {
+            const int key = 16 * ts + 8 * jh + vkey0, col = 32 * (pt * DBP + db) + vcol0;
+            const int addr = key * ROWB + (((col >> 3) ^ v_swz<D>(key)) * 16) + (col & 7) * 2;
+            const short4v rr = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (short4v __attribute__((address_space(3)))*)(lds_v + addr));
+            const uintx2 r2 = __builtin_bit_cast(uintx2, rr);
+            a[2 * jh] = r2[0]; a[2 * jh + 1] = r2[1];
+          }
+          if constexpr (BF16 && !PB) a = bf16x8_to_f16x8(a);
+          vfr[ts][db] = a;
         }
-        if constexpr (BF16 && !PB) a = bf16x8_to_f16x8(a);
-        vfr[ts][db] = a;
+      if (pt == PORTIONS - 1) {
+        lds_wait();
+        __syncthreads();                            // both wavefronts hold their V fragments: the V buffer is free
+        if (has1) v_copy(cxn & COL_MASK);
       }
-    lds_wait();
-    __syncthreads();                                // both wavefronts hold their V fragments: the V buffer is free
-    if (has1) v_copy(cxn & COL_MASK);
-    // ---- O^T += V^T P^T ----
 #pragma unroll
-    for (int ts = 0; ts < 4; ++ts)
+      for (int ts = 0; ts < 4; ++ts)
 #pragma unroll
-      for (int db = 0; db < DB; ++db)
-        oacc[db][0] = mfma_qk<PB>(vfr[ts][db], pf[ts][0], oacc[db][0]);
+        for (int db = 0; db < DBP; ++db)
+          oacc[pt * DBP + db][0] = mfma_qk<PB>(vfr[ts][db], pf[ts][0], oacc[pt * DBP + db][0]);
+    }
     if (has1) {
       wait_vm<VOPS>();                              // this wavefront's half of K(t+1) has landed (V(t+1) may be in flight)
       __syncthreads();                              // ... and the other half
@@ -266,30 +282,36 @@ __global__ __launch_bounds__(128, 2) void fwd_pair_kernel(const FwdParams prm) {
         lsum > 0.f ? (m_i + __builtin_amdgcn_logf(lsum)) * 0.6931471805599453f : -INFINITY;
 }
 
-template <int DT, bool EW>
+template <int D, int DT, bool EW>
 static void launch_pair_t(const FwdParams& prm, hipStream_t st) {
   static bool configured = false;
   if (!configured) {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_pair_kernel<DT, EW>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, PAIR_LDS_BYTES);
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_pair_kernel<D, DT, EW>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, pair_lds_bytes<D>());
     configured = true;
   }
   const int BH = prm.B * prm.H;
   const int grid = ((BH + 7) / 8) * 8 * prm.nb;
-  hipLaunchKernelGGL((fwd_pair_kernel<DT, EW>), dim3(grid), dim3(128), PAIR_LDS_BYTES, st, prm);
+  hipLaunchKernelGGL((fwd_pair_kernel<D, DT, EW>), dim3(grid), dim3(128), pair_lds_bytes<D>(), st, prm);
 }
 
-// D = 128 only.  dt: 0 fp16, 1 bf16 with P rounded to fp16 (V converted), 2 bf16 with P rounded to bf16.
-void launch_fwd_pair(const FwdParams& prm, int dt, bool elementwise, hipStream_t st) {
+template <int D>
+static void launch_pair_d(const FwdParams& prm, int dt, bool elementwise, hipStream_t st) {
   if (!elementwise) {
-    if (dt == 0) launch_pair_t<0, false>(prm, st);
-    else if (dt == 1) launch_pair_t<1, false>(prm, st);
-    else launch_pair_t<2, false>(prm, st);
+    if (dt == 0) launch_pair_t<D, 0, false>(prm, st);
+    else if (dt == 1) launch_pair_t<D, 1, false>(prm, st);
+    else launch_pair_t<D, 2, false>(prm, st);
   } else {
-    if (dt == 0) launch_pair_t<0, true>(prm, st);
-    else if (dt == 1) launch_pair_t<1, true>(prm, st);
-    else launch_pair_t<2, true>(prm, st);
+    if (dt == 0) launch_pair_t<D, 0, true>(prm, st);
+    else if (dt == 1) launch_pair_t<D, 1, true>(prm, st);
+    else launch_pair_t<D, 2, true>(prm, st);
   }
+}
+
+// D: 128 or 256.  dt: 0 fp16, 1 bf16 with P rounded to fp16 (V converted), 2 bf16 with P rounded to bf16.
+void launch_fwd_pair(const FwdParams& prm, int D, int dt, bool elementwise, hipStream_t st) {
+  if (D == 128) launch_pair_d<128>(prm, dt, elementwise, st);
+  else launch_pair_d<256>(prm, dt, elementwise, st);
 }
 
 }  // namespace bsattn

@@ -89,6 +89,7 @@ __device__ __forceinline__ uintx4 bf16x8_to_f16x8(uintx4 x) {
 //  K tile: operand reads take one chunk of 32 consecutive rows -> spread the chunk index over rows.
 //  V tile: transpose reads take 64 contiguous bytes of 4 consecutive rows -> move rows to
 //          different 64-byte parts of the 256-byte bank period.
+// (D = 256: the D = 128 patterns on the low four bits of the 32 chunk indices of a row)
 template <int D> __device__ __forceinline__ int k_swz(int row) { return D == 64 ? ((row >> 1) & 7) : (row & 15); }
 template <int D> __device__ __forceinline__ int v_swz(int row) { return D == 64 ? (((row >> 1) & 1) << 2) : ((row & 3) << 2); }
 
@@ -148,7 +149,7 @@ __device__ __forceinline__ void store_out4(void* obase, int64_t elem_off, bool o
 // Swizzle for tiles that are read both ways (operand reads of 32 consecutive rows and
 // transpose reads of 4 consecutive rows x 64 bytes): a bijection of the row bits that
 // separates both access patterns over the 64 LDS banks.
-template <int D> __device__ __forceinline__ int u_swz(int row) {
+template <int D> __device__ __forceinline__ int u_swz(int row) {   // (D = 256 as D = 128, on the low four chunk bits)
   if (D == 64) { const int x = (row >> 1) & 7; return ((x & 1) << 2) | (x >> 1); }
   return ((row & 3) << 2) | ((row >> 2) & 3);
 }

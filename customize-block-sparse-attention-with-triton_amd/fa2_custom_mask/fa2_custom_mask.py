@@ -41,8 +41,8 @@ def _check_qkv(q, k, v, mask):
     if q.dtype not in (torch.float16, torch.bfloat16) or k.dtype != q.dtype or v.dtype != q.dtype:
         raise TypeError("q, k, v must all be float16 or all bfloat16")
     B, H, N, D = q.shape
-    if D not in (16, 32, 64, 128):                                     # :58 and fa2_fwd.py:120 (256 is not built)
-        raise ValueError("head dimension must be 16, 32, 64 or 128")
+    if D not in (16, 32, 64, 128, 256):                                # :58
+        raise ValueError("head dimension must be 16, 32, 64, 128 or 256")
     if N < 1:
         raise ValueError("empty sequence")
     if mask is None:
@@ -195,8 +195,8 @@ def flash_attention_custom_mask(q, k, v, mask=None, sm_scale=1.3):
     """Drop-in for the reference's `flash_attention_custom_mask = _attention.apply`
     (fa2_custom_mask.py:157): q,k,v [B,H,N,D] fp16/bf16 on the GPU, mask bool
     [B|1,H|1,nb,nb] with nb = ceil(N/64) (or elementwise [B|1,H|1,N,N]; None = dense attention),
-    returns o like q.  D is 16, 32, 64 or 128; N need not be a multiple of 64 (the last block of a
-    block mask then covers the remaining tokens).  Shapes other than D in {64,128}, N % 64 == 0
+    returns o like q.  D is 16, 32, 64, 128 or 256; N need not be a multiple of 64 (the last block of a
+    block mask then covers the remaining tokens).  Shapes other than D in {64,128,256}, N % 64 == 0
     cost one zero-padded copy of q, k, v per call.  The kept-tile lists of a mask tensor are cached
     until the tensor is modified."""
     return _attention.apply(q, k, v, mask, sm_scale)

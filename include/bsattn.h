@@ -35,7 +35,7 @@ extern "C" {
 #define BSATTN_ERR_NULL (-1)       /* a required pointer is NULL */
 #define BSATTN_ERR_SHAPE (-2)      /* non-positive size, N not a multiple of 64, bad broadcast */
 #define BSATTN_ERR_DTYPE (-3)      /* unknown dtype code */
-#define BSATTN_ERR_HEAD_DIM (-4)   /* head dimension not in {64, 128} */
+#define BSATTN_ERR_HEAD_DIM (-4)   /* head dimension not in {64, 128, 256} */
 #define BSATTN_ERR_STRIDE (-5)     /* innermost stride != 1 or rows not 16-byte aligned */
 #define BSATTN_ERR_WORKSPACE (-6)  /* workspace NULL or too small */
 #define BSATTN_ERR_LAUNCH (-7)     /* the HIP runtime refused a launch */

@@ -45,7 +45,7 @@ def test_argument_validation_without_gpu():
     assert fwd(q=None) == -1 and fwd(rp=None) == -1
     assert fwd(N=100) == -2 and fwd(B=0) == -2 and fwd(Bm=3, B=2) == -2
     assert fwd(dt=5) == -3 and fwd(odt=1) == -3
-    assert fwd(D=96) == -4 and fwd(D=256) == -4
+    assert fwd(D=96) == -4 and fwd(D=512) == -4
     bad = (ctypes.c_int64 * 4)(64 * 64, 64 * 64, 64, 2)
     assert fwd(qs=bad) == -5
     odd = (ctypes.c_int64 * 4)(64 * 68, 64 * 68, 68, 1)

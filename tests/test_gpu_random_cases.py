@@ -20,7 +20,7 @@ pytestmark = pytest.mark.gpu
 
 def draw_case(seed):
     rs = np.random.RandomState(seed)
-    D = int(rs.choice([16, 32, 64, 64, 128, 128]))
+    D = int(rs.choice([16, 32, 64, 64, 128, 128, 256]))
     dtype = torch.float16 if rs.rand() < 0.5 else torch.bfloat16
     B, H = int(rs.choice([1, 1, 2, 3])), int(rs.choice([1, 2, 4, 8]))
     if rs.rand() < 0.15:

@@ -104,9 +104,44 @@ def test_tail_words_bit_exact(dev):
         assert np.array_equal(bits[:T].cpu().numpy().view(np.uint64), w_ref)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_head_dim_256(dev, dtype):
+    """D = 256 (fa2_custom_mask.py:58 lists it): forward, LSE and gradients against the oracle, block mask, elementwise
+    mask with partly set tiles and queries without keys, a sequence length that is not a multiple of 64, and a
+    launch with few row blocks (row and column lists shared between workgroups in the backward)."""
+    block = uniform_block_mask(1, 2, 8, 0.5, 90)
+    block[0, 0, 3, :] = False
+    check(dev, 1, 2, 512, 256, dtype, block, cut_mask(block, 512), 91)
+    g = torch.Generator().manual_seed(92)
+    m = (torch.rand(1, 1, 200, 200, generator=g) < 0.4) & torch.tril(torch.ones(200, 200, dtype=torch.bool))
+    m[0, 0, 9, :] = False
+    check(dev, 2, 3, 200, 256, dtype, m, m.numpy(), 93)
+    long_block = uniform_block_mask(1, 1, 32, 0.6, 94)
+    check(dev, 1, 1, 2048, 256, dtype, long_block, cut_mask(long_block, 2048), 95)
+
+
+def test_head_dim_256_bf16_typed_results_many_heads(dev):
+    import fa2_custom_mask as fm
+    B, H, N, D = 2, 32, 256, 256
+    q, k, v, do = make_qkv(B, H, N, D, torch.bfloat16, 96, n=4)
+    block = uniform_block_mask(1, 1, 4, 0.7, 97)
+    sc = 1.0 / 16.0
+    o, lse, dq, dk, dv = fm.attention_forward_backward(q.to(dev), k.to(dev), v.to(dev), block.to(dev), sc, do.to(dev))
+    torch.cuda.synchronize()
+    for hd in (0, 63):
+        b, h = divmod(hd, H)
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        o_ref = orc.naive_attention(f32(q[sl]), f32(k[sl]), f32(v[sl]), cut_mask(block, N), sc)
+        refs = orc.attention_backward(f32(q[sl]), f32(k[sl]), f32(v[sl]), cut_mask(block, N), sc, f32(do[sl]))
+        for got, ref in ((o, o_ref), (dq, refs[0]), (dk, refs[1]), (dv, refs[2])):
+            assert got.dtype == torch.bfloat16
+            ma, rl = errors(got[sl], ref)
+            assert ma <= 3e-2 and rl <= 4e-3
+
+
 def test_unsupported_head_dim_is_an_error(dev):
     import fa2_custom_mask as fm
-    q = torch.zeros(1, 1, 128, 256, dtype=torch.float16, device=dev)
+    q = torch.zeros(1, 1, 128, 512, dtype=torch.float16, device=dev)
     with pytest.raises(ValueError):
         fm.flash_attention_custom_mask(q, q, q, None, 0.1)
     q = torch.zeros(1, 1, 128, 48, dtype=torch.float16, device=dev)
