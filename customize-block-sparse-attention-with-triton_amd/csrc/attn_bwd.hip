@@ -339,6 +339,7 @@ __global__ __launch_bounds__(128, (QB == 1 && D == 64) ? 2 : 1) void dkdv_kernel
   constexpr int KS = D / 16, STEPS = 2 / QB;
   constexpr int DB = DH < 0 ? D / 32 : D / 64, DB0 = DH < 0 ? 0 : DH * DB;   // 32-column blocks of this launch, the first one
   constexpr int PORTIONS = D == 256 ? 2 : 1, KSP = KS / PORTIONS;            // fragments of the first products in portions
+  static_assert(QB == 1 || PORTIONS == 1, "whole tiles per step only without portions");
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
   const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int ln = lane & 31, g = lane >> 5;
@@ -405,76 +406,171 @@ __global__ __launch_bounds__(128, (QB == 1 && D == 64) ? 2 : 1) void dkdv_kernel
     const float* st_lse = reinterpret_cast<const float*>(gt + C::TILE_BYTES) + qoff;
     const float* st_dlt = st_lse + 64;
 
-    // operand fragments are read from LDS ahead of the block of MFMAs that consumes them
-    floatx16 sacc[QB], dpacc[QB];
+    if constexpr (QB == 2) {
+      // Whole tile per step, one query block after the other, so that the vector work on one query
+      // block (P and dS) sits beside matrix work on the other: scores of block 0; scores of block 1
+      // beside P, dS of block 0; second products of block 0 beside P, dS of block 1; second
+      // products of block 1.
+      floatx16 sacc[2], dpacc[2];
+      uintx4 pf[4], dsf[4];
+      uintx4 fq[KS], fg[KS];
+      auto read_rows = [&](int qb) {
 #pragma unroll
-    for (int qb = 0; qb < QB; ++qb) { sacc[qb] = zero16(); dpacc[qb] = zero16(); }
+        for (int s = 0; s < KS; ++s) {
+          fq[s] = frag_rows<D>(qt, 32 * qb, s, ln, g);
+          fg[s] = frag_rows<D>(gt, 32 * qb, s, ln, g);
+        }
+      };
+      auto first = [&](int qb) {
+        sacc[qb] = zero16(); dpacc[qb] = zero16();
 #pragma unroll
-    for (int pt = 0; pt < PORTIONS; ++pt) {
-      uintx4 fq[QB][KSP], fg[QB][KSP];
+        for (int s = 0; s < KS; ++s) {
+          sacc[qb] = mfma_qk<BF16>(fq[s], kfr[s], sacc[qb]);      // S = Q K^T
+          dpacc[qb] = mfma_qk<BF16>(fg[s], vfr[s], dpacc[qb]);    // dP = dO V^T
+        }
+      };
+      unsigned long long mw = 0ull;
+      if constexpr (EW)
+        mw = *reinterpret_cast<const unsigned long long*>(gt + C::TILE_BYTES + C::STAT_BYTES + (32 * wv + ln) * 8) >> (4 * g);
+      auto p_and_ds = [&](int qb) {          // rows of the results are queries: register i <-> query 32qb + 8(i/4) + 4g + i%4
+        if constexpr (EW) mask_scores(sacc[qb], (unsigned)(mw >> (32 * qb)));
 #pragma unroll
-      for (int s = 0; s < KSP; ++s)
+        for (int t2 = 0; t2 < 2; ++t2)
 #pragma unroll
-        for (int qb = 0; qb < QB; ++qb) {
-          fq[qb][s] = frag_rows<D>(qt, 32 * qb, pt * KSP + s, ln, g);
-          fg[qb][s] = frag_rows<D>(gt, 32 * qb, pt * KSP + s, ln, g);
+          for (int jh = 0; jh < 2; ++jh) {
+            const int ts = 2 * qb + t2, i0 = 8 * t2 + 4 * jh;
+            const int q0 = 32 * qb + 8 * (i0 >> 2) + 4 * g;
+            const floatx4 l4 = *reinterpret_cast<const floatx4*>(st_lse + q0);
+            const floatx4 d4 = *reinterpret_cast<const floatx4*>(st_dlt + q0);
+            float p[4], ds[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float nl = EW && l4[e] == -INFINITY ? -INFINITY : -l4[e] * kLog2e;
+              p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[qb][i0 + e], qk_scale, nl));
+              ds[e] = p[e] * (dpacc[qb][i0 + e] - d4[e]);
+            }
+            pf[ts][2 * jh] = pack2<PB>(p[0], p[1]);   pf[ts][2 * jh + 1] = pack2<PB>(p[2], p[3]);
+            dsf[ts][2 * jh] = pack2<PB>(ds[0], ds[1]); dsf[ts][2 * jh + 1] = pack2<PB>(ds[2], ds[3]);
+          }
+      };
+      uintx4 fgt[2][DB], fqt[2][DB];
+      auto read_cols = [&](int qb) {
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+          for (int db = 0; db < DB; ++db) {
+            fgt[t2][db] = frag_cols<D, BF16 && !PB>(gt, DB0 + db, 2 * qb + t2, lane);
+            fqt[t2][db] = frag_cols<D, BF16 && !PB>(qt, DB0 + db, 2 * qb + t2, lane);
+          }
+      };
+      auto second = [&](int qb) {
+#pragma unroll
+        for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+          for (int db = 0; db < DB; ++db) {
+            dvacc[db] = mfma_qk<PB>(fgt[t2][db], pf[2 * qb + t2], dvacc[db]);    // dV^T += dO^T P
+            dkacc[db] = mfma_qk<PB>(fqt[t2][db], dsf[2 * qb + t2], dkacc[db]);   // dK^T += Q^T dS
+          }
+      };
+      read_rows(0);
+      __builtin_amdgcn_sched_barrier(0);
+      first(0);
+      __builtin_amdgcn_sched_barrier(0);
+      read_rows(1);
+      read_cols(0);
+      __builtin_amdgcn_sched_barrier(0);
+      first(1);
+      p_and_ds(0);
+#pragma unroll
+      for (int it = 0; it < 2 * KS; ++it) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      second(0);
+      p_and_ds(1);
+#pragma unroll
+      for (int it = 0; it < 4 * DB; ++it) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      read_cols(1);
+      __builtin_amdgcn_sched_barrier(0);
+      second(1);
+    } else {
+      // operand fragments are read from LDS ahead of the block of MFMAs that consumes them
+      floatx16 sacc[QB], dpacc[QB];
+  #pragma unroll
+      for (int qb = 0; qb < QB; ++qb) { sacc[qb] = zero16(); dpacc[qb] = zero16(); }
+  #pragma unroll
+      for (int pt = 0; pt < PORTIONS; ++pt) {
+        uintx4 fq[QB][KSP], fg[QB][KSP];
+  #pragma unroll
+        for (int s = 0; s < KSP; ++s)
+  #pragma unroll
+          for (int qb = 0; qb < QB; ++qb) {
+            fq[qb][s] = frag_rows<D>(qt, 32 * qb, pt * KSP + s, ln, g);
+            fg[qb][s] = frag_rows<D>(gt, 32 * qb, pt * KSP + s, ln, g);
+          }
+        __builtin_amdgcn_sched_barrier(0);
+  #pragma unroll
+        for (int s = 0; s < KSP; ++s)
+  #pragma unroll
+          for (int qb = 0; qb < QB; ++qb) {
+            sacc[qb] = mfma_qk<BF16>(fq[qb][s], kfr[pt * KSP + s], sacc[qb]);      // S = Q K^T
+            dpacc[qb] = mfma_qk<BF16>(fg[qb][s], vfr[pt * KSP + s], dpacc[qb]);    // dP = dO V^T
+          }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (EW) {
+        unsigned long long mw = *reinterpret_cast<const unsigned long long*>(
+            gt + C::TILE_BYTES + C::STAT_BYTES + (32 * wv + ln) * 8);
+        if constexpr (QB == 1) mw >>= qoff;
+        mw >>= 4 * g;
+        if constexpr (QB == 2) mask_scores(sacc[0], sacc[1], mw);
+        else mask_scores(sacc[0], (unsigned)mw);
+      }
+      // dO^T and Q^T fragments of the second products, read under the exponentials below
+      uintx4 fgt[2 * QB][DB], fqt[2 * QB][DB];
+  #pragma unroll
+      for (int ts = 0; ts < 2 * QB; ++ts)
+  #pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          fgt[ts][db] = frag_cols<D, BF16 && !PB>(gt, DB0 + db, ts, lane);
+          fqt[ts][db] = frag_cols<D, BF16 && !PB>(qt, DB0 + db, ts, lane);
         }
       __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int s = 0; s < KSP; ++s)
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb) {
-          sacc[qb] = mfma_qk<BF16>(fq[qb][s], kfr[pt * KSP + s], sacc[qb]);      // S = Q K^T
-          dpacc[qb] = mfma_qk<BF16>(fg[qb][s], vfr[pt * KSP + s], dpacc[qb]);    // dP = dO V^T
+      // rows of the results are queries: register i of block qb <-> query 32qb + 8(i/4) + 4g + i%4
+      uintx4 pf[2 * QB], dsf[2 * QB];
+  #pragma unroll
+      for (int ts = 0; ts < 2 * QB; ++ts)
+  #pragma unroll
+        for (int jh = 0; jh < 2; ++jh) {
+          const int qb = ts >> 1, i0 = 8 * (ts & 1) + 4 * jh;
+          const int q0 = 32 * qb + 8 * (i0 >> 2) + 4 * g;
+          const floatx4 l4 = *reinterpret_cast<const floatx4*>(st_lse + q0);
+          const floatx4 d4 = *reinterpret_cast<const floatx4*>(st_dlt + q0);
+          float p[4], ds[4];
+  #pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            // (a query without any unmasked key has lse = -inf: its P must come out as 0)
+            const float nl = EW && l4[e] == -INFINITY ? -INFINITY : -l4[e] * kLog2e;
+            p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[qb][i0 + e], qk_scale, nl));
+            ds[e] = p[e] * (dpacc[qb][i0 + e] - d4[e]);
+          }
+          pf[ts][2 * jh] = pack2<PB>(p[0], p[1]);   pf[ts][2 * jh + 1] = pack2<PB>(p[2], p[3]);
+          dsf[ts][2 * jh] = pack2<PB>(ds[0], ds[1]); dsf[ts][2 * jh + 1] = pack2<PB>(ds[2], ds[3]);
         }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    if constexpr (EW) {
-      unsigned long long mw = *reinterpret_cast<const unsigned long long*>(
-          gt + C::TILE_BYTES + C::STAT_BYTES + (32 * wv + ln) * 8);
-      if constexpr (QB == 1) mw >>= qoff;
-      mw >>= 4 * g;
-      if constexpr (QB == 2) mask_scores(sacc[0], sacc[1], mw);
-      else mask_scores(sacc[0], (unsigned)mw);
-    }
-    // dO^T and Q^T fragments of the second products, read under the exponentials below
-    uintx4 fgt[2 * QB][DB], fqt[2 * QB][DB];
-#pragma unroll
-    for (int ts = 0; ts < 2 * QB; ++ts)
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        fgt[ts][db] = frag_cols<D, BF16 && !PB>(gt, DB0 + db, ts, lane);
-        fqt[ts][db] = frag_cols<D, BF16 && !PB>(qt, DB0 + db, ts, lane);
-      }
-    __builtin_amdgcn_sched_barrier(0);
-    // rows of the results are queries: register i of block qb <-> query 32qb + 8(i/4) + 4g + i%4
-    uintx4 pf[2 * QB], dsf[2 * QB];
-#pragma unroll
-    for (int ts = 0; ts < 2 * QB; ++ts)
-#pragma unroll
-      for (int jh = 0; jh < 2; ++jh) {
-        const int qb = ts >> 1, i0 = 8 * (ts & 1) + 4 * jh;
-        const int q0 = 32 * qb + 8 * (i0 >> 2) + 4 * g;
-        const floatx4 l4 = *reinterpret_cast<const floatx4*>(st_lse + q0);
-        const floatx4 d4 = *reinterpret_cast<const floatx4*>(st_dlt + q0);
-        float p[4], ds[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          // (a query without any unmasked key has lse = -inf: its P must come out as 0)
-          const float nl = EW && l4[e] == -INFINITY ? -INFINITY : -l4[e] * kLog2e;
-          p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[qb][i0 + e], qk_scale, nl));
-          ds[e] = p[e] * (dpacc[qb][i0 + e] - d4[e]);
+  #pragma unroll
+      for (int ts = 0; ts < 2 * QB; ++ts)
+  #pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          dvacc[db] = mfma_qk<PB>(fgt[ts][db], pf[ts], dvacc[db]);    // dV^T += dO^T P
+          dkacc[db] = mfma_qk<PB>(fqt[ts][db], dsf[ts], dkacc[db]);   // dK^T += Q^T dS
         }
-        pf[ts][2 * jh] = pack2<PB>(p[0], p[1]);   pf[ts][2 * jh + 1] = pack2<PB>(p[2], p[3]);
-        dsf[ts][2 * jh] = pack2<PB>(ds[0], ds[1]); dsf[ts][2 * jh + 1] = pack2<PB>(ds[2], ds[3]);
-      }
-#pragma unroll
-    for (int ts = 0; ts < 2 * QB; ++ts)
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        dvacc[db] = mfma_qk<PB>(fgt[ts][db], pf[ts], dvacc[db]);    // dV^T += dO^T P
-        dkacc[db] = mfma_qk<PB>(fqt[ts][db], dsf[ts], dkacc[db]);   // dK^T += Q^T dS
-      }
+  
+    }
   }
 
   if (prm.split > 1) {   // unscaled fp32 parts; sum_parts_kernel adds them up
