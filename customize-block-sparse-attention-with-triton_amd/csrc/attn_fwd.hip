@@ -798,11 +798,13 @@ static unsigned long long next_epoch() {
 }
 
 int compute_units() {
+  static int cached[64] = {0};   // per device; the value never changes, so a race only repeats the query
   int dev = 0, cus = 256;
-  if (hipGetDevice(&dev) == hipSuccess) {
-    int v = 0;
-    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
-  }
+  if (hipGetDevice(&dev) != hipSuccess) return cus;
+  if (dev >= 0 && dev < 64 && cached[dev] > 0) return cached[dev];
+  int v = 0;
+  if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) cus = v;
+  if (dev >= 0 && dev < 64) cached[dev] = cus;
   return cus;
 }
 
