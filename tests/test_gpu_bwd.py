@@ -87,3 +87,19 @@ def test_invariant_rowsum_ds_zero(dev):
     _, _, dq, dk, dv = fm.attention_forward_backward(q.to(dev), k.to(dev), vc.to(dev), mask.to(dev), 0.125,
                                                      do.to(dev), out_fp32=True)
     assert float(dq.abs().max()) <= 2e-3 and float(dk.abs().max()) <= 2e-3
+
+
+def test_strided_inputs_backward(dev):
+    """q, k, v as views of one packed [B, N, 3, H, D] tensor (what a fused projection produces) and a
+    strided dO: gradients equal those of contiguous copies bit for bit (no atomics anywhere)."""
+    import fa2_custom_mask as fm
+    B, H, N, D = 2, 3, 256, 64
+    g = torch.Generator().manual_seed(21)
+    qkv = torch.randn(B, N, 3, H, D, generator=g).to(torch.float16).to(dev)
+    q, k, v = [qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3)]
+    do = torch.randn(B, N, H, D, generator=g).to(torch.float16).to(dev).permute(0, 2, 1, 3)
+    m = uniform_block_mask(1, 1, N // 64, 0.6, 22).to(dev)
+    res_s = fm.attention_forward_backward(q, k, v, m, 0.125, do)
+    res_c = fm.attention_forward_backward(q.contiguous(), k.contiguous(), v.contiguous(), m, 0.125, do.contiguous())
+    for a, b_ in zip(res_s[2:], res_c[2:]):
+        assert torch.equal(a, b_)
