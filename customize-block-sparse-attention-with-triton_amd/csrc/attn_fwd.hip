@@ -823,8 +823,24 @@ static size_t slots_bytes(int B, int H, int W, int D) {
   return (size_t)B * H * W * partial_floats(D) * sizeof(float);
 }
 
+// Pair kernel: workgroups per row block.  One when the launch has enough row blocks to fill the GPU twice
+// over; otherwise the row lists are shared (up to 8 ways, a share of a dense list keeping at least 8 tiles).
+static int pair_split(int B, int H, int nb, int D) {
+  const int64_t row_blocks = (int64_t)B * H * nb;
+  const int64_t want = (int64_t)compute_units() * (D == 128 ? 4 : 2) * 2;
+  if (row_blocks >= want) return 1;
+  int64_t s = (want + row_blocks - 1) / row_blocks;
+  const int cap = nb / 8 > 1 ? nb / 8 : 1;
+  if (s > cap) s = cap;
+  return (int)(s > 8 ? 8 : s);
+}
+
+static size_t pair_parts_bytes(int B, int H, int N, int D, int split) {
+  return split > 1 ? (size_t)split * B * H * N * (D + 2) * sizeof(float) : 0;
+}
+
 size_t fwd_workspace_bytes(int B, int H, int N, int D) {
-  if (D == 256) return 256;     // one wavefront pair per row block: nothing is shared between workgroups
+  if (D == 256) return 256 + pair_parts_bytes(B, H, N, D, pair_split(B, H, N / 64, D));   // the pair kernel only
   const int nb = N / 64;
   const int W = groups_per_head(B, H, nb, D);
   return slots_bytes(B, H, W, D) + (size_t)B * H * W * sizeof(unsigned long long);
@@ -882,7 +898,14 @@ int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
   for (int i = 0; i < 3; ++i) { prm.qs[i] = s.qs[i]; prm.ks[i] = s.ks[i]; prm.vs[i] = s.vs[i]; prm.os[i] = s.os[i]; }
   const bool bf = s.dtype == BSATTN_BF16;
   const int BH = s.B * s.H;
+  prm.split = 1;
   if (s.D == 256 || (s.D == 128 && use_pair_kernel((int64_t)BH * prm.nb, prm.nb))) {   // (D = 256 has no other kernel)
+    // D = 256 launches with few row blocks share the row lists between workgroups; at D = 128 the
+    // cooperative kernel below takes those launches (sharing was measured: faster on dense masks with 2-3
+    // heads, 25-30 % slower on sparse ones)
+    if (s.D == 256) prm.split = pair_split(s.B, s.H, prm.nb, s.D);
+    prm.part_o = (float*)ws + 64;
+    prm.part_ml = prm.part_o + (size_t)prm.split * BH * s.N * s.D;
     launch_fwd_pair(prm, s.D, !bf ? 0 : (prm.out_f32 ? 1 : 2), tile_bits != nullptr, st);
     return launch_status();
   }

@@ -40,8 +40,10 @@ __global__ __launch_bounds__(128, D == 128 ? 2 : 1) void fwd_pair_kernel(const F
   const int nb = prm.nb, BH = prm.B * prm.H;
   // linear id -> (head, row block): groups of 8 heads, one head per XCD, long row blocks first
   int bh, m;
+  const int per_chunk = gridDim.x / prm.split;    // chunk = slowest index: head i of a group stays on XCD i
+  const int chunk = blockIdx.x / per_chunk;
   {
-    const int L = blockIdx.x;
+    const int L = blockIdx.x - chunk * per_chunk;
     const int grp = L / (8 * nb), l = L - grp * 8 * nb;
     const int hg = BH - 8 * grp < 8 ? BH - 8 * grp : 8;
     bh = 8 * grp + l % hg;
@@ -51,7 +53,13 @@ __global__ __launch_bounds__(128, D == 128 ? 2 : 1) void fwd_pair_kernel(const F
   const int b = bh / prm.H, h = bh % prm.H;
   const int mh = (prm.Bm > 1 ? b : 0) * prm.Hm + (prm.Hm > 1 ? h : 0);
   const cint_ptr_t rp = (cint_ptr_t)(uintptr_t)(prm.row_ptr + (int64_t)mh * nb);
-  const int t0 = rp[m], t1 = rp[m + 1];
+  int t0 = rp[m], t1 = rp[m + 1];
+  if (prm.split > 1) {                           // this workgroup's share of the row block's list
+    const int len = t1 - t0;
+    t1 = t0 + (int)((int64_t)len * (chunk + 1) / prm.split);
+    t0 = t0 + (int)((int64_t)len * chunk / prm.split);
+    if (t0 == t1) return;                        // (pair_sum_parts_kernel knows which shares are empty)
+  }
   void* obase = out_base(prm, b, h);
   const int64_t qrow = (int64_t)m * 64 + 32 * w + ln;          // this lane's query
   if (t0 == t1) {                                // no kept tile: O = 0, lse = -inf
@@ -270,6 +278,20 @@ __global__ __launch_bounds__(128, D == 128 ? 2 : 1) void fwd_pair_kernel(const F
 
   // ---- normalise and write ----
   const float lsum = l_i + __shfl_xor(l_i, 32);
+  if (prm.split > 1) {   // unnormalised fp32 part with its reference exponent and row sum
+    float* part = prm.part_o + ((int64_t)chunk * BH + bh) * prm.N * D;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4)
+        store_out4<BF16>(part, qrow * D + 32 * db + 8 * i4 + 4 * g, true, oacc[db][0][4 * i4], oacc[db][0][4 * i4 + 1],
+                         oacc[db][0][4 * i4 + 2], oacc[db][0][4 * i4 + 3]);
+    if (g == 0) {
+      float* ml = prm.part_ml + (((int64_t)chunk * BH + bh) * prm.N + qrow) * 2;
+      ml[0] = m_i; ml[1] = lsum;
+    }
+    return;
+  }
   const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
 #pragma unroll
   for (int db = 0; db < DB; ++db)
@@ -282,6 +304,44 @@ __global__ __launch_bounds__(128, D == 128 ? 2 : 1) void fwd_pair_kernel(const F
         lsum > 0.f ? (m_i + __builtin_amdgcn_logf(lsum)) * 0.6931471805599453f : -INFINITY;
 }
 
+// split > 1: O = sum_c 2^(m_c - M) O_c / sum_c 2^(m_c - M) l_c over the non-empty shares c of a row block
+// (M = max m_c over shares with mass), lse = (M + log2 of the denominator) ln 2.  One thread per 4
+// consecutive output values.
+template <bool BF16>
+__global__ __launch_bounds__(256) void pair_sum_parts_kernel(const FwdParams prm, int D, int64_t quads) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= quads) return;
+  const int qpr = D / 4;                                     // threads per query row
+  const int64_t rowg = i / qpr;                              // row over all heads
+  const int col = (int)(i % qpr) * 4;
+  const int bh = (int)(rowg / prm.N), row = (int)(rowg % prm.N);
+  const int b = bh / prm.H, h = bh % prm.H, BH = prm.B * prm.H;
+  const int mh = (prm.Bm > 1 ? b : 0) * prm.Hm + (prm.Hm > 1 ? h : 0);
+  const int32_t* rp = prm.row_ptr + (int64_t)mh * prm.nb;
+  const int t0 = rp[row / 64], len = rp[row / 64 + 1] - t0;
+  float M = -INFINITY;
+  for (int c = 0; c < prm.split; ++c) {
+    if ((int64_t)len * c / prm.split == (int64_t)len * (c + 1) / prm.split) continue;      // empty share: nothing was written
+    const float* ml = prm.part_ml + (((int64_t)c * BH + bh) * prm.N + row) * 2;
+    if (ml[1] > 0.f) M = fmaxf(M, ml[0]);
+  }
+  float L = 0.f;
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int c = 0; c < prm.split; ++c) {
+    if ((int64_t)len * c / prm.split == (int64_t)len * (c + 1) / prm.split) continue;
+    const float* ml = prm.part_ml + (((int64_t)c * BH + bh) * prm.N + row) * 2;
+    if (!(ml[1] > 0.f)) continue;
+    const float wgt = __builtin_amdgcn_exp2f(ml[0] - M);
+    L += wgt * ml[1];
+    acc += wgt * *reinterpret_cast<const floatx4*>(prm.part_o + (((int64_t)c * BH + bh) * prm.N + row) * D + col);
+  }
+  const float inv = L > 0.f ? 1.0f / L : 0.f;
+  store_out4<BF16>(out_base(prm, b, h), (int64_t)row * prm.os[2] + col, prm.out_f32, acc[0] * inv, acc[1] * inv, acc[2] * inv,
+                   acc[3] * inv);
+  if (col == 0 && prm.lse != nullptr)
+    prm.lse[(int64_t)bh * prm.N + row] = L > 0.f ? (M + __builtin_amdgcn_logf(L)) * 0.6931471805599453f : -INFINITY;
+}
+
 template <int D, int DT, bool EW>
 static void launch_pair_t(const FwdParams& prm, hipStream_t st) {
   static bool configured = false;
@@ -291,8 +351,12 @@ static void launch_pair_t(const FwdParams& prm, hipStream_t st) {
     configured = true;
   }
   const int BH = prm.B * prm.H;
-  const int grid = ((BH + 7) / 8) * 8 * prm.nb;
+  const int grid = ((BH + 7) / 8) * 8 * prm.nb * prm.split;
   hipLaunchKernelGGL((fwd_pair_kernel<D, DT, EW>), dim3(grid), dim3(128), pair_lds_bytes<D>(), st, prm);
+  if (prm.split > 1) {
+    const int64_t quads = (int64_t)BH * prm.N * D / 4;
+    hipLaunchKernelGGL((pair_sum_parts_kernel<DT != 0>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, st, prm, D, quads);
+  }
 }
 
 template <int D>

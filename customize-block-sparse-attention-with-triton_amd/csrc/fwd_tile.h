@@ -14,6 +14,8 @@ struct FwdParams {
   float* ws;                       // partial slots of row blocks shared between workgroups
   unsigned long long* flags;       // one per slot: holds `epoch` once the slot's part is complete
   unsigned long long epoch;        // distinguishes this launch's flags from stale contents
+  int split;                       // pair kernel: workgroups per row block (1: results written directly)
+  float* part_o; float* part_ml;   // split > 1: unnormalised fp32 O parts [split][B*H][N][D] and their (m, l) [split][B*H][N][2]
   int B, H, N, nb, Bm, Hm, W;   // W: workgroups per head
   int first_ids;                // workgroups with a linear id below this are the first on their compute unit
   int out_f32;

@@ -104,8 +104,8 @@ class ForwardPlan:
 
     def __init__(self, q, k, v, lists, sm_scale, out_dtype=None, stream=None):
         B, H, N, D = q.shape
-        if N % TILE or D not in (64, 128):
-            raise ValueError("a plan takes whole tiles only: N % 64 == 0 and D in {64, 128}")
+        if N % TILE or D not in (64, 128, 256):
+            raise ValueError("a plan takes whole tiles only: N % 64 == 0 and D in {64, 128, 256}")
         self.q, self.k, self.v, self.lists = _prep(q), _prep(k), _prep(v), lists
         out_dtype = out_dtype or q.dtype
         self.o = torch.empty((B, H, N, D), dtype=out_dtype, device=q.device)
