@@ -68,6 +68,18 @@ def test_very_long_sequence_n262144(dev):
     assert float(np.abs(o[0, 0, 2001 * 64:2002 * 64]).max()) == 0.0
 
 
+def test_head_dim_256_row_lists_shared_by_workgroups(dev):
+    """D = 256, one head, 128 row blocks: every row list is split over 8 workgroups whose fp32 parts a
+    second kernel sums.  Rows with fewer tiles than parts (empty parts), a full row and an empty row."""
+    nb = 128
+    mask = uniform_block_mask(1, 1, nb, 0.04, 1241)
+    mask[0, 0, 5, :] = True
+    mask[0, 0, 6, :] = False
+    mask[0, 0, 7, :] = False; mask[0, 0, 7, 100] = True
+    q, k, v, o = sampled_forward_check(dev, nb * 64, 256, mask, 1241, [0, 5, 7, 64, 127])
+    assert float(np.abs(o[0, 0, 6 * 64:7 * 64]).max()) == 0.0
+
+
 def test_c2_dense_elementwise_mask_n6400(dev):
     """C2: preprocessing from a dense N x N bool mask (tile-constant) feeds the same result."""
     import fa2_custom_mask as fm
