@@ -647,8 +647,8 @@ static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
   // 32 keys are 192 registers) and halves were measured slower (718 against 688 us, C5).
   constexpr int QB = D == 128 ? 2 : 1;   // (D = 256: halves, and the head dimension of dK, dV in two launches)
   using CK = BwdCfg<D, EW, 32 * QB>;
-  static bool configured = false;   // raising the dynamic LDS limit is idempotent
-  if (!configured) {
+  static std::atomic<unsigned long long> configured{0};   // raising the dynamic LDS limit is idempotent
+  once_per_device(configured, [] {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dq_kernel<D, BF16, EW, PB, KB>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, CQ::LDS_BYTES);
     if constexpr (D == 256) {
@@ -660,8 +660,7 @@ static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
       (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv_kernel<D, BF16, EW, PB, QB, -1>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, CK::LDS_BYTES);
     }
-    configured = true;
-  }
+  });
   const int BH = prm.B * prm.H;
   constexpr int RPB = 256 / (D / 8);
   hipLaunchKernelGGL((delta_kernel<D, BF16>), dim3((prm.N + RPB - 1) / RPB, BH), dim3(256), 0, st, prm);

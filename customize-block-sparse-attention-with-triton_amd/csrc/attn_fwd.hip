@@ -865,14 +865,13 @@ static bool rows_mode(const FwdParams& prm) { return prm.nb >= 8 * prm.W; }
 template <int D, int DT, bool EW>
 static void launch_fwd_t(const FwdParams& prm, int BH, hipStream_t st) {
   using C = FwdCfg<D>;
-  static bool configured = false;   // raising the dynamic LDS limit is idempotent
-  if (!configured) {
+  static std::atomic<unsigned long long> configured{0};   // raising the dynamic LDS limit is idempotent
+  once_per_device(configured, [] {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<D, DT, false, EW>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<D, DT, true, EW>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-    configured = true;
-  }
+  });
   if (rows_mode(prm)) {
     hipLaunchKernelGGL((fwd_kernel<D, DT, true, EW>), dim3(prm.W * BH), dim3(C::NW * 64), C::LDS_BYTES, st, prm);
   } else {

@@ -344,12 +344,11 @@ __global__ __launch_bounds__(256) void pair_sum_parts_kernel(const FwdParams prm
 
 template <int D, int DT, bool EW>
 static void launch_pair_t(const FwdParams& prm, hipStream_t st) {
-  static bool configured = false;
-  if (!configured) {
+  static std::atomic<unsigned long long> configured{0};   // raising the dynamic LDS limit is idempotent
+  once_per_device(configured, [] {
     (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_pair_kernel<D, DT, EW>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, pair_lds_bytes<D>());
-    configured = true;
-  }
+  });
   const int BH = prm.B * prm.H;
   const int grid = ((BH + 7) / 8) * 8 * prm.nb * prm.split;
   hipLaunchKernelGGL((fwd_pair_kernel<D, DT, EW>), dim3(grid), dim3(128), pair_lds_bytes<D>(), st, prm);

@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <atomic>
 #include "bsattn.h"
 
 #define BSATTN_VERSION 100
@@ -30,6 +31,19 @@ struct AttnShape {
 
 // attn_fwd.hip
 int compute_units();   // of the current device (256 if the query fails)
+
+// Runs f unless it has completed before for the current device (one `done` mask per call site):
+// kernel attributes such as the dynamic LDS limit are kept per device.  Two threads may both run
+// f for a device; f must be idempotent.
+template <class F>
+inline void once_per_device(std::atomic<unsigned long long>& done, F&& f) {
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  const unsigned long long bit = 1ull << (dev & 63);
+  if (done.load(std::memory_order_acquire) & bit) return;
+  f();
+  done.fetch_or(bit, std::memory_order_release);
+}
 size_t fwd_workspace_bytes(int B, int H, int N, int D);
 int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                const int32_t* row_ptr, const int32_t* col_idx, const uint8_t* tile_partial,
