@@ -18,6 +18,9 @@
 #include "fwd_tile.h"
 #include "kernel_util.h"
 
+#ifndef PAIR_EARLY_V
+#define PAIR_EARLY_V 1   // largest number of fragment portions (head dimension / 128) for which V is read early
+#endif
 namespace bsattn {
 
 constexpr int PAIR_COLS_CAP = 1024;                               // column indices of the row block kept in LDS
@@ -225,22 +228,13 @@ __global__ __launch_bounds__(128, D == 128 ? 2 : 1) void fwd_pair_kernel(const F
         }
       }
     }
-    // ---- softmax numerators ----
     uintx4 pf[4][2];
-    float lnew = softmax_tile<FOLD, PB>(s0, s1, qk_scale, m_i, l_i, pf, 0);
-    if (__any(fresh || (EW && l_i == 0.f) || !(lnew - l_i < 16384.0f))) {
-      recentre<DB, FOLD, EW>(s0, s1, oacc, 0, qk_scale, m_i, l_i, mfrag, fresh, g);
-      lnew = softmax_tile<FOLD, PB>(s0, s1, qk_scale, m_i, l_i, pf, 0);
-    }
-    l_i = lnew;
-    fresh = false;
     // ---- V^T fragments ----
-    if (has1) wait_vm<KOPS>(); else wait_vm<0>();   // this wavefront's half of V(t) has landed (K(t+1) may be in flight)
-    if (t > t0) __syncthreads();                    // ... and the other half (the first tile was waited for above)
-    // ---- O^T += V^T P^T, the V^T fragments taken in PORTIONS portions ----
-#pragma unroll
-    for (int pt = 0; pt < PORTIONS; ++pt) {
-      uintx4 vfr[4][DBP];
+    auto v_landed = [&]() {
+      if (has1) wait_vm<KOPS>(); else wait_vm<0>();   // this wavefront's half of V(t) has landed (K(t+1) may be in flight)
+      if (t > t0) __syncthreads();                    // ... and the other half (the first tile was waited for above)
+    };
+    auto read_v = [&](int pt, uintx4 (&vfr)[4][DBP]) {
 #pragma unroll
       for (int ts = 0; ts < 4; ++ts)
 #pragma unroll
@@ -258,16 +252,50 @@ __global__ __launch_bounds__(128, D == 128 ? 2 : 1) void fwd_pair_kernel(const F
           if constexpr (BF16 && !PB) a = bf16x8_to_f16x8(a);
           vfr[ts][db] = a;
         }
-      if (pt == PORTIONS - 1) {
-        lds_wait();
-        __syncthreads();                            // both wavefronts hold their V fragments: the V buffer is free
-        if (has1) v_copy(cxn & COL_MASK);
-      }
+    };
+    auto v_free = [&]() {
+      lds_wait();
+      __syncthreads();                            // both wavefronts hold their V fragments: the V buffer is free
+      if (has1) v_copy(cxn & COL_MASK);
+    };
+    auto second = [&](int pt, uintx4 (&vfr)[4][DBP]) {
 #pragma unroll
       for (int ts = 0; ts < 4; ++ts)
 #pragma unroll
         for (int db = 0; db < DBP; ++db)
           oacc[pt * DBP + db][0] = mfma_qk<PB>(vfr[ts][db], pf[ts][0], oacc[pt * DBP + db][0]);
+    };
+    auto numerators = [&]() {
+      float lnew = softmax_tile<FOLD, PB>(s0, s1, qk_scale, m_i, l_i, pf, 0);
+      if (__any(fresh || (EW && l_i == 0.f) || !(lnew - l_i < 16384.0f))) {
+        recentre<DB, FOLD, EW>(s0, s1, oacc, 0, qk_scale, m_i, l_i, mfrag, fresh, g);
+        lnew = softmax_tile<FOLD, PB>(s0, s1, qk_scale, m_i, l_i, pf, 0);
+      }
+      l_i = lnew;
+      fresh = false;
+    };
+    if constexpr (PORTIONS <= PAIR_EARLY_V) {
+      // The V fragments are read before the softmax (they take the registers of the K fragments), so
+      // that the next V tile is requested that much earlier: its latency was exposed otherwise.
+      uintx4 vfr[PORTIONS][4][DBP];
+      v_landed();
+#pragma unroll
+      for (int pt = 0; pt < PORTIONS; ++pt) read_v(pt, vfr[pt]);
+      v_free();
+      numerators();
+#pragma unroll
+      for (int pt = 0; pt < PORTIONS; ++pt) second(pt, vfr[pt]);
+    } else {
+      numerators();
+      v_landed();
+      // ---- O^T += V^T P^T, the V^T fragments taken in PORTIONS portions ----
+#pragma unroll
+      for (int pt = 0; pt < PORTIONS; ++pt) {
+        uintx4 vfr[4][DBP];
+        read_v(pt, vfr);
+        if (pt == PORTIONS - 1) v_free();
+        second(pt, vfr);
+      }
     }
     if (has1) {
       wait_vm<VOPS>();                              // this wavefront's half of K(t+1) has landed (V(t+1) may be in flight)
