@@ -46,7 +46,6 @@ def event_times(fn, iters, warmup, torch):
 
 def fwd_bwd_c5(torch, dev, fm, steps, warmup):
     """HIP-event times of one forward call and one backward call at configs[4]."""
-    from fa2_custom_mask import fa2_custom_mask as host
     B, H, Nc, Dc = 2, 16, 8192, 128
     nbc = Nc // TILE
     g = torch.Generator().manual_seed(1238)
@@ -57,16 +56,18 @@ def fwd_bwd_c5(torch, dev, fm, steps, warmup):
     lists_t = fm.block_mask_to_lists(m, transpose=True)
     tiles = int(lists.counts[1]) * B * H
     sc = 1.0 / Dc ** 0.5
-    o, lse = host._forward(q, k, v, lists, sc, torch.bfloat16, True)
-    tf = event_times(lambda: host._forward(q, k, v, lists, sc, torch.bfloat16, True), steps, warmup, torch)
-    tb = event_times(lambda: host._backward(q, k, v, o, do, lse, lists, lists_t, sc, torch.bfloat16), steps, warmup, torch)
+    fplan = fm.ForwardPlan(q, k, v, lists, sc)
+    o, lse = fplan.run()
+    bplan = fm.BackwardPlan(q, k, v, o, do, lse, lists, lists_t, sc)
+    tf = event_times(fplan.run, steps, warmup, torch)
+    tb = event_times(bplan.run, steps, warmup, torch)
     mf, mb = tf[len(tf) // 2], tb[len(tb) // 2]
     ff, fb = tiles * 4.0 * TILE * TILE * Dc, tiles * 10.0 * TILE * TILE * Dc
     return {"workload": "BASELINE configs[4]: fwd+bwd B=2 H=16 N=8192 D=128 bf16, block-causal keep 0.25 shared mask",
             "kept_tiles": tiles, "fwd_ms": round(mf, 5), "fwd_tflops": round(ff / mf / 1e9, 1),
             "bwd_ms": round(mb, 5), "bwd_tflops": round(fb / mb / 1e9, 1),
             "frac_mfma_peak": {"fwd": round(ff / mf / 1e9 / PEAK_F16_TFLOPS, 4), "bwd": round(fb / mb / 1e9 / PEAK_F16_TFLOPS, 4)},
-            "note": "times include the per-call output/workspace allocation of the host wrapper"}
+            "note": "one bsattn_fwd call and one bsattn_bwd call (delta, dq and dkdv kernels), buffers allocated beforehand"}
 
 
 def elementwise_case(torch, dev, fm, q, k, v, sm_scale):

@@ -151,6 +151,40 @@ def _backward(q, k, v, o, do, lse, lists, lists_t, sm_scale, out_dtype):
     return dq, dk, dv
 
 
+class BackwardPlan:
+    """The backward counterpart of ForwardPlan: dq, dk, dv and the workspace allocated once, the C
+    arguments marshalled once; run() only enqueues the kernels.  o and lse are the forward's
+    results for the same q, k, v; block masks only."""
+
+    def __init__(self, q, k, v, o, do, lse, lists, lists_t, sm_scale, out_dtype=None, stream=None):
+        B, H, N, D = q.shape
+        if N % TILE or D not in (64, 128, 256) or lists.bits is not None:
+            raise ValueError("a plan takes whole tiles and block masks only: N % 64 == 0 and D in {64, 128, 256}")
+        self.q, self.k, self.v, self.o, self.do = _prep(q), _prep(k), _prep(v), _prep(o), _prep(do)
+        self.lse, self.lists, self.lists_t = lse, lists, lists_t
+        out_dtype = out_dtype or q.dtype
+        self.dq = torch.empty((B, H, N, D), dtype=out_dtype, device=q.device)
+        self.dk = torch.empty_like(self.dq)
+        self.dv = torch.empty_like(self.dq)
+        wsb = _ext.bwd_workspace(B, H, N, D)
+        self.ws = torch.empty(wsb, dtype=torch.uint8, device=q.device)
+        self._keep = tuple(_ext.strides4(t) for t in (self.q, self.k, self.v, self.o, self.do))
+        stream = stream if stream is not None else torch.cuda.current_stream(q.device)
+        self._args = (self.q.data_ptr(), self.k.data_ptr(), self.v.data_ptr(), self.o.data_ptr(), self.do.data_ptr(),
+                      lse.data_ptr(), self.dq.data_ptr(), self.dk.data_ptr(), self.dv.data_ptr(),
+                      lists.row_ptr.data_ptr(), lists.col_idx.data_ptr(), lists_t.row_ptr.data_ptr(),
+                      lists_t.col_idx.data_ptr(), lists.Bm, lists.Hm, B, H, N, D, _ext.dtype_code(q.dtype),
+                      _ext.dtype_code(out_dtype), float(sm_scale)) + self._keep + (
+                          self.ws.data_ptr(), wsb, ctypes.c_void_p(stream.cuda_stream))
+        self._fn = _ext.lib().bsattn_bwd
+
+    def run(self):
+        rc = self._fn(*self._args)
+        if rc != 0:
+            _ext.check(rc, "bsattn_bwd")
+        return self.dq, self.dk, self.dv
+
+
 class _attention(torch.autograd.Function):
     """forward(q, k, v, mask, sm_scale) as the reference (fa2_custom_mask.py:43-94); two extra
     trailing arguments select an fp32 output and the LSE as second result."""

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from oracle import bsattn_oracle as orc
-from helpers import make_qkv, uniform_block_mask, causal_block_mask, errors, f32
+from helpers import make_qkv, uniform_block_mask, causal_block_mask, errors, f32, same_up_to_rounding
 
 pytestmark = pytest.mark.gpu
 MAXABS = {torch.float16: 2e-2, torch.bfloat16: 3e-2}
@@ -106,3 +106,29 @@ def test_strided_inputs_backward(dev):
     from helpers import same_up_to_rounding
     for a, b_ in zip(res_s[2:], res_c[2:]):
         assert same_up_to_rounding(a, b_, rel=2.0 ** -8, abs_=2e-3)
+
+
+def test_backward_plan_matches_the_call(dev):
+    """BackwardPlan (buffers and arguments prepared once) against attention_forward_backward, run
+    twice on a workspace filled with ones in between (split lists: fp32 parts in the workspace)."""
+    import fa2_custom_mask as fm
+    B, H, N, D = 1, 2, 2048, 128
+    q, k, v, do = [x.to(dev) for x in make_qkv(B, H, N, D, torch.bfloat16, 611, n=4)]
+    mask = causal_block_mask(1, 1, N // 64, 0.5, 612).to(dev)
+    sc = 1.0 / np.sqrt(D)
+    o, lse, dq, dk, dv = fm.attention_forward_backward(q, k, v, mask, sc, do)
+    lists = fm.block_mask_to_lists(mask)
+    lists_t = fm.block_mask_to_lists(mask, transpose=True)
+    plan = fm.BackwardPlan(q, k, v, o, do, lse, lists, lists_t, sc)
+    for fill in (None, 255):
+        if fill is not None:
+            plan.ws.fill_(fill)
+        for t in (plan.dq, plan.dk, plan.dv):
+            t.fill_(float("nan"))
+        got = plan.run()
+        torch.cuda.synchronize()
+        for a, b_ in zip(got, (dq, dk, dv)):
+            assert same_up_to_rounding(a, b_, rel=2.0 ** -8, abs_=2e-3)
+    with pytest.raises(ValueError):
+        fm.BackwardPlan(q[:, :, :100], k[:, :, :100], v[:, :, :100], o[:, :, :100], do[:, :, :100], lse[:, :, :100],
+                        lists, lists_t, sc)
