@@ -23,9 +23,9 @@ PEAK_F16_TFLOPS = 2500.0     # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0
 SEED = 1234 + 2
 # HBM-side bytes of one keep-1.0 forward launch, from two rocprofv3 --pmc runs (FETCH_SIZE x 2.0 and
-# WRITE_SIZE x 1.0 after scaling by the readings of a 256 MiB device copy): 226863 KiB fetched +
-# 18899 KiB written.
-TRAFFIC_BYTES_PER_LAUNCH = (226863 + 18899) * 1024
+# WRITE_SIZE x 1.0 after scaling by the readings of a 256 MiB device copy): 204792 KiB fetched +
+# 11334 KiB written.
+TRAFFIC_BYTES_PER_LAUNCH = (204792 + 11334) * 1024
 
 
 def tile_flops(kept):
@@ -292,7 +292,7 @@ def main():
         "token_reorder": reorder_case(torch, dev, fm),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "fwd_kernel<64, 0, false, false> (fp16, one bsattn_fwd call)",
+                     "kernel": "fwd_kernel<64, 0, false, false, true> (fp16, contiguous rows, one bsattn_fwd call)",
                      "algorithmic_flops_per_launch": tile_flops(kept[1.0])},
     }
     if not args.no_cpu:

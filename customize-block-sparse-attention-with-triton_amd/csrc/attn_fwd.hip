@@ -64,7 +64,8 @@ template <int D> struct FwdCfg {
 };
 
 // DT: 0 fp16; 1 bf16 with P rounded to fp16 (V fragments converted); 2 bf16 with P rounded to bf16.
-template <int D, int DT, bool ROWS, bool EW>
+// CONTIG: the rows of K and of V follow each other without gaps (row stride = D).
+template <int D, int DT, bool ROWS, bool EW, bool CONTIG>
 __global__ __launch_bounds__(FwdCfg<D>::NW * 64, FwdCfg<D>::WG_PER_CU)
 void fwd_kernel(const FwdParams prm) {
   constexpr bool BF16 = DT != 0, PB = DT == 2;
@@ -150,9 +151,26 @@ void fwd_kernel(const FwdParams prm) {
   const unsigned long long* lds_bits = reinterpret_cast<const unsigned long long*>(lds + C::BITS_OFF + w * 512);
   constexpr int KOPS = CPR + (EW ? 2 : 0);      // instructions of one K copy
   // copy of the K tile `tile` = entry t of the kept-tile list (EW: with its 512 bytes of mask words)
+  // CONTIG (rows that follow each other without gaps, the usual case): copy instruction j reads at
+  // byte offset 1024 j from the tile and writes at 1024 j from the buffer, and the instruction's immediate
+  // offset applies to both, so four instructions share one scalar base and one m0 (6 instead of 24 scalar
+  // instructions per tile copy at D = 64).
+  constexpr bool k_contig = CONTIG, v_contig = CONTIG;
+  auto copy4 = [&](const unsigned short* src, unsigned o0, unsigned o1, unsigned o2, unsigned o3, unsigned dst) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %5\n\tglobal_load_lds_dwordx4 %2, %5 offset:1024\n\t"
+                 "global_load_lds_dwordx4 %3, %5 offset:2048\n\tglobal_load_lds_dwordx4 %4, %5 offset:3072"
+                 :: "s"(dst), "v"(o0), "v"(o1), "v"(o2), "v"(o3), "s"(src) : "memory", "m0");
+  };
   auto k_copy_all = [&](const unsigned short* tile, int t) {
+    if constexpr (k_contig) {
 #pragma unroll
-    for (int j = 0; j < CPR; ++j) k_copy(tile, j);
+      for (int jb = 0; jb < CPR; jb += 4)
+        copy4(tile + jb * RPI * D, koff[jb % KPER], koff[(jb + 1) % KPER], koff[(jb + 2) % KPER], koff[(jb + 3) % KPER],
+              lds_k_addr + jb * 1024);
+    } else {
+#pragma unroll
+      for (int j = 0; j < CPR; ++j) k_copy(tile, j);
+    }
     if constexpr (EW) {
       const unsigned long long* src = prm.tile_bits + (int64_t)t * 64;
 #pragma unroll
@@ -162,8 +180,14 @@ void fwd_kernel(const FwdParams prm) {
     }
   };
   auto v_copy_all = [&](const unsigned short* tile) {
+    if constexpr (v_contig) {
 #pragma unroll
-    for (int j = 0; j < CPR; ++j) v_copy(tile, j);
+      for (int jb = 0; jb < CPR; jb += 4)
+        copy4(tile + jb * RPI * D, voff[0], voff[0], voff[0], voff[0], lds_v_addr + jb * 1024);
+    } else {
+#pragma unroll
+      for (int j = 0; j < CPR; ++j) v_copy(tile, j);
+    }
   };
   // per-lane LDS byte offsets of the operand reads.  K fragment (kb, s): row 32kb+ln, chunk 2s+g
   int kaddr[2][KS];
@@ -872,21 +896,29 @@ static bool use_pair_kernel(int64_t row_blocks, int nb) {
 // wavefront takes whole row blocks, which needs no merge and no second kernel.
 static bool rows_mode(const FwdParams& prm) { return prm.nb >= 8 * prm.W; }
 
-template <int D, int DT, bool EW>
-static void launch_fwd_t(const FwdParams& prm, int BH, hipStream_t st) {
+template <int D, int DT, bool EW, bool CONTIG>
+static void launch_fwd_c(const FwdParams& prm, int BH, hipStream_t st) {
   using C = FwdCfg<D>;
   static std::atomic<unsigned long long> configured{0};   // raising the dynamic LDS limit is idempotent
   once_per_device(configured, [] {
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<D, DT, false, EW>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<D, DT, false, EW, CONTIG>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<D, DT, true, EW>),
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<D, DT, true, EW, CONTIG>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
   });
   if (rows_mode(prm)) {
-    hipLaunchKernelGGL((fwd_kernel<D, DT, true, EW>), dim3(prm.W * BH), dim3(C::NW * 64), C::LDS_BYTES, st, prm);
+    hipLaunchKernelGGL((fwd_kernel<D, DT, true, EW, CONTIG>), dim3(prm.W * BH), dim3(C::NW * 64), C::LDS_BYTES, st, prm);
   } else {
-    hipLaunchKernelGGL((fwd_kernel<D, DT, false, EW>), dim3(prm.W * BH), dim3(C::NW * 64), C::LDS_BYTES, st, prm);
+    hipLaunchKernelGGL((fwd_kernel<D, DT, false, EW, CONTIG>), dim3(prm.W * BH), dim3(C::NW * 64), C::LDS_BYTES, st, prm);
   }
+}
+
+// The copies with immediate offsets are compiled for D = 64 only (2-4 % there; every variant doubles the
+// number of kernels).
+template <int D, int DT, bool EW>
+static void launch_fwd_t(const FwdParams& prm, int BH, hipStream_t st) {
+  if (D == 64 && prm.ks[2] == D && prm.vs[2] == D) launch_fwd_c<D, DT, EW, D == 64>(prm, BH, st);
+  else launch_fwd_c<D, DT, EW, false>(prm, BH, st);
 }
 
 int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
