@@ -156,6 +156,7 @@ void fwd_kernel(const FwdParams prm) {
   // offset applies to both, so four instructions share one scalar base and one m0 (6 instead of 24 scalar
   // instructions per tile copy at D = 64).
   constexpr bool k_contig = CONTIG, v_contig = CONTIG;
+  const int64_t k_rs = CONTIG ? (int64_t)D : prm.ks[2], v_rs = CONTIG ? (int64_t)D : prm.vs[2];   // row strides (a constant: a tile's address is a shift)
   auto copy4 = [&](const unsigned short* src, unsigned o0, unsigned o1, unsigned o2, unsigned o3, unsigned dst) {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %5\n\tglobal_load_lds_dwordx4 %2, %5 offset:1024\n\t"
                  "global_load_lds_dwordx4 %3, %5 offset:2048\n\tglobal_load_lds_dwordx4 %4, %5 offset:3072"
@@ -337,7 +338,7 @@ void fwd_kernel(const FwdParams prm) {
     }
     lds_wait();      // the K fragments have arrived: the K buffer is free
     mid();
-    if (has1) k_copy_all(kg + (int64_t)cbn * 64 * prm.ks[2], tn);
+    if (has1) k_copy_all(kg + (int64_t)cbn * 64 * k_rs, tn);
     auto mask_scores = [&](floatx16& s0, floatx16& s1, unsigned long long mw) {
       const unsigned lo = (unsigned)mw, hi = (unsigned)(mw >> 32);
 #pragma unroll
@@ -371,7 +372,7 @@ void fwd_kernel(const FwdParams prm) {
       read_v();
     }
     lds_wait();      // the V fragments have arrived: the V buffer is free
-    if (copy_v) v_copy_all(vg + (int64_t)cbn * 64 * prm.vs[2]);
+    if (copy_v) v_copy_all(vg + (int64_t)cbn * 64 * v_rs);
     // [3]
     second(0);
     float lnew1 = softmax_tile<FOLD, PB>(sb0, sb1, qk_scale, m_i[1], l_i[1], pf, 1);
@@ -462,8 +463,8 @@ void fwd_kernel(const FwdParams prm) {
       if (ta < tb) {
         int cx = __builtin_amdgcn_readfirstlane(col_of(ta));      // current tile: column block | flag
         if (kdone != ta) {
-          k_copy_all(kg + (int64_t)(cx & COL_MASK) * 64 * prm.ks[2], ta);
-          v_copy_all(vg + (int64_t)(cx & COL_MASK) * 64 * prm.vs[2]);
+          k_copy_all(kg + (int64_t)(cx & COL_MASK) * 64 * k_rs, ta);
+          v_copy_all(vg + (int64_t)(cx & COL_MASK) * 64 * v_rs);
         }
         reset_acc();
         load_q(row);
@@ -607,8 +608,8 @@ void fwd_kernel(const FwdParams prm) {
       reset_acc();
       if (mine) {
         int cx = __builtin_amdgcn_readfirstlane(col_of(cur));     // current tile: column block | flag
-        if (kdone != cur) { k_copy_all(kg + (int64_t)(cx & COL_MASK) * 64 * prm.ks[2], cur); kdone = cur; }
-        if (vdone != cur) { v_copy_all(vg + (int64_t)(cx & COL_MASK) * 64 * prm.vs[2]); vdone = cur; }
+        if (kdone != cur) { k_copy_all(kg + (int64_t)(cx & COL_MASK) * 64 * k_rs, cur); kdone = cur; }
+        if (vdone != cur) { v_copy_all(vg + (int64_t)(cx & COL_MASK) * 64 * v_rs); vdone = cur; }
         load_q(r);
         while (cur < seg_b) {
           // draw the tile after next; the value is picked up inside the tile
