@@ -157,16 +157,11 @@ void fwd_kernel(const FwdParams prm) {
   // instructions per tile copy at D = 64).
   constexpr bool k_contig = CONTIG, v_contig = CONTIG;
   const int64_t k_rs = CONTIG ? (int64_t)D : prm.ks[2], v_rs = CONTIG ? (int64_t)D : prm.vs[2];   // row strides (a constant: a tile's address is a shift)
-  auto copy4 = [&](const unsigned short* src, unsigned o0, unsigned o1, unsigned o2, unsigned o3, unsigned dst) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %5\n\tglobal_load_lds_dwordx4 %2, %5 offset:1024\n\t"
-                 "global_load_lds_dwordx4 %3, %5 offset:2048\n\tglobal_load_lds_dwordx4 %4, %5 offset:3072"
-                 :: "s"(dst), "v"(o0), "v"(o1), "v"(o2), "v"(o3), "s"(src) : "memory", "m0");
-  };
   auto k_copy_all = [&](const unsigned short* tile, int t) {
     if constexpr (k_contig) {
 #pragma unroll
       for (int jb = 0; jb < CPR; jb += 4)
-        copy4(tile + jb * RPI * D, koff[jb % KPER], koff[(jb + 1) % KPER], koff[(jb + 2) % KPER], koff[(jb + 3) % KPER],
+        tile_load_async_four(tile + jb * RPI * D, koff[jb % KPER], koff[(jb + 1) % KPER], koff[(jb + 2) % KPER], koff[(jb + 3) % KPER],
               lds_k_addr + jb * 1024);
     } else {
 #pragma unroll
@@ -184,7 +179,7 @@ void fwd_kernel(const FwdParams prm) {
     if constexpr (v_contig) {
 #pragma unroll
       for (int jb = 0; jb < CPR; jb += 4)
-        copy4(tile + jb * RPI * D, voff[0], voff[0], voff[0], voff[0], lds_v_addr + jb * 1024);
+        tile_load_async_four(tile + jb * RPI * D, voff[0], voff[0], voff[0], voff[0], lds_v_addr + jb * 1024);
     } else {
 #pragma unroll
       for (int j = 0; j < CPR; ++j) v_copy(tile, j);

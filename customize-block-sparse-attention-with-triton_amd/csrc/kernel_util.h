@@ -118,6 +118,16 @@ __device__ __forceinline__ void tile_load_async_one(const unsigned short* tile, 
   asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(lds_addr), "v"(off), "s"(tile) : "memory", "m0");
 }
 
+// Four consecutive instructions of a tile copy whose rows follow each other without gaps: the
+// immediate offset of the instruction applies to the source and to the LDS address alike, so the
+// four share one scalar base and one m0.
+__device__ __forceinline__ void tile_load_async_four(const unsigned short* src, unsigned o0, unsigned o1, unsigned o2,
+                                                     unsigned o3, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %5\n\tglobal_load_lds_dwordx4 %2, %5 offset:1024\n\t"
+               "global_load_lds_dwordx4 %3, %5 offset:2048\n\tglobal_load_lds_dwordx4 %4, %5 offset:3072"
+               :: "s"(lds_addr), "v"(o0), "v"(o1), "v"(o2), "v"(o3), "s"(src) : "memory", "m0");
+}
+
 template <int N> __device__ __forceinline__ void wait_vm() {
   asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
 }
