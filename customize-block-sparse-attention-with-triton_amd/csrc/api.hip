@@ -20,6 +20,7 @@ const char* bsattn_strerror(int code) {
     case BSATTN_ERR_WORKSPACE: return "workspace missing or too small";
     case BSATTN_ERR_LAUNCH: return "HIP launch failed";
     case BSATTN_ERR_RANGE: return "size exceeds 32-bit index range";
+    case BSATTN_ERR_STATIC_LIMIT: return "shape needs more scratch memory than the library's static buffer holds";
     default: return "unknown error code";
   }
 }
@@ -104,12 +105,11 @@ int bsattn_fwd_workspace(int B, int H, int N, int D, size_t* bytes) {
   return BSATTN_OK;
 }
 
-static int fwd_common(const void* q, const void* k, const void* v, void* o, float* lse,
-                      const int32_t* row_ptr, const int32_t* col_idx, const uint8_t* tile_partial,
-                      const uint64_t* tile_bits, int Bm, int Hm, int B, int H, int N,
-                      int D, int dtype, int out_dtype, float sm_scale, const int64_t* q_strides,
-                      const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides,
-                      void* workspace, size_t workspace_bytes, void* stream) {
+// Everything bsattn_fwd and its variants check before the workspace question.
+static int fwd_check(const void* q, const void* k, const void* v, void* o, const int32_t* row_ptr,
+                     const int32_t* col_idx, int Bm, int Hm, int B, int H, int N, int D, int dtype,
+                     int out_dtype, const int64_t* q_strides, const int64_t* k_strides,
+                     const int64_t* v_strides, const int64_t* o_strides) {
   if (q == nullptr || k == nullptr || v == nullptr || o == nullptr || row_ptr == nullptr || col_idx == nullptr)
     return BSATTN_ERR_NULL;
   int rc = check_attn(Bm, Hm, B, H, N, D, dtype, out_dtype);
@@ -117,7 +117,18 @@ static int fwd_common(const void* q, const void* k, const void* v, void* o, floa
   if ((rc = check_strides(q_strides, 2, q)) != BSATTN_OK) return rc;
   if ((rc = check_strides(k_strides, 2, k)) != BSATTN_OK) return rc;
   if ((rc = check_strides(v_strides, 2, v)) != BSATTN_OK) return rc;
-  if ((rc = check_strides(o_strides, out_dtype == BSATTN_F32 ? 4 : 2, o)) != BSATTN_OK) return rc;
+  return check_strides(o_strides, out_dtype == BSATTN_F32 ? 4 : 2, o);
+}
+
+static int fwd_common(const void* q, const void* k, const void* v, void* o, float* lse,
+                      const int32_t* row_ptr, const int32_t* col_idx, const uint8_t* tile_partial,
+                      const uint64_t* tile_bits, int Bm, int Hm, int B, int H, int N,
+                      int D, int dtype, int out_dtype, float sm_scale, const int64_t* q_strides,
+                      const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides,
+                      void* workspace, size_t workspace_bytes, void* stream) {
+  const int rc = fwd_check(q, k, v, o, row_ptr, col_idx, Bm, Hm, B, H, N, D, dtype, out_dtype, q_strides, k_strides,
+                           v_strides, o_strides);
+  if (rc != BSATTN_OK) return rc;
   if (workspace == nullptr || workspace_bytes < fwd_workspace_bytes(B, H, N, D)) return BSATTN_ERR_WORKSPACE;
   AttnShape s;
   s.B = B; s.H = H; s.N = N; s.D = D; s.Bm = Bm; s.Hm = Hm; s.dtype = dtype; s.out_dtype = out_dtype;
@@ -133,6 +144,22 @@ int bsattn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                void* workspace, size_t workspace_bytes, void* stream) {
   return fwd_common(q, k, v, o, lse, row_ptr, col_idx, nullptr, nullptr, Bm, Hm, B, H, N, D, dtype, out_dtype,
                     sm_scale, q_strides, k_strides, v_strides, o_strides, workspace, workspace_bytes, stream);
+}
+
+int bsattn_fwd_static(const void* q, const void* k, const void* v, void* o, float* lse,
+                      const int32_t* row_ptr, const int32_t* col_idx, int Bm, int Hm, int B, int H, int N,
+                      int D, int dtype, int out_dtype, float sm_scale, const int64_t* q_strides,
+                      const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides,
+                      void* stream) {
+  int rc = fwd_check(q, k, v, o, row_ptr, col_idx, Bm, Hm, B, H, N, D, dtype, out_dtype, q_strides, k_strides,
+                     v_strides, o_strides);
+  if (rc != BSATTN_OK) return rc;
+  const size_t need = fwd_workspace_bytes(B, H, N, D);
+  if (need > (size_t)BSATTN_STATIC_SCRATCH_BYTES) return BSATTN_ERR_STATIC_LIMIT;
+  void* ws = nullptr;
+  if ((rc = static_scratch(&ws)) != BSATTN_OK) return rc;
+  return fwd_common(q, k, v, o, lse, row_ptr, col_idx, nullptr, nullptr, Bm, Hm, B, H, N, D, dtype, out_dtype,
+                    sm_scale, q_strides, k_strides, v_strides, o_strides, ws, need, stream);
 }
 
 int bsattn_fwd_elementwise(const void* q, const void* k, const void* v, void* o, float* lse,

@@ -918,6 +918,26 @@ static void launch_fwd_t(const FwdParams& prm, int BH, hipStream_t st) {
   else launch_fwd_c<D, DT, EW, false>(prm, BH, st);
 }
 
+// ---- forward without any allocation by anybody: the scratch memory is part of the library ----
+// A file-scope device array stands in for the workspace argument of launch_fwd.  In host code its name
+// is only a handle: the address the kernels may use is asked for once per device (each device holds
+// its own copy of the array at its own address).
+static __device__ __align__(256) unsigned char scratch[BSATTN_STATIC_SCRATCH_BYTES];
+
+int static_scratch(void** ptr) {
+  static std::atomic<void*> per_device[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return BSATTN_ERR_LAUNCH;
+  void* p = per_device[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    // (two threads may both ask: they get the same answer)
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return BSATTN_ERR_LAUNCH;
+    per_device[dev].store(p, std::memory_order_release);
+  }
+  *ptr = p;
+  return BSATTN_OK;
+}
+
 int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                const int32_t* row_ptr, const int32_t* col_idx, const uint8_t* tile_partial,
                const uint64_t* tile_bits, const AttnShape& s, void* ws, hipStream_t st) {

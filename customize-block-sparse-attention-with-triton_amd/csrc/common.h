@@ -48,6 +48,8 @@ size_t fwd_workspace_bytes(int B, int H, int N, int D);
 int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                const int32_t* row_ptr, const int32_t* col_idx, const uint8_t* tile_partial,
                const uint64_t* tile_bits, const AttnShape& s, void* ws, hipStream_t st);
+// Address, on the current device, of the library's own scratch array (BSATTN_STATIC_SCRATCH_BYTES).
+int static_scratch(void** ptr);
 
 // attn_bwd.hip
 size_t bwd_workspace_bytes(int B, int H, int N, int D);

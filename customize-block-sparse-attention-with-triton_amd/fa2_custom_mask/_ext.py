@@ -29,6 +29,8 @@ _SIGNATURES = {
     "bsattn_fwd_workspace": ([_i, _i, _i, _i, ctypes.POINTER(ctypes.c_size_t)], _i),
     "bsattn_fwd": ([_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f,
                     _p, _p, _p, _p, _p, ctypes.c_size_t, _p], _i),
+    "bsattn_fwd_static": ([_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f,
+                           _p, _p, _p, _p, _p], _i),
     "bsattn_fwd_elementwise": ([_p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f,
                                 _p, _p, _p, _p, _p, ctypes.c_size_t, _p], _i),
     "bsattn_bwd_workspace": ([_i, _i, _i, _i, ctypes.POINTER(ctypes.c_size_t)], _i),

@@ -40,6 +40,8 @@ extern "C" {
 #define BSATTN_ERR_WORKSPACE (-6)  /* workspace NULL or too small */
 #define BSATTN_ERR_LAUNCH (-7)     /* the HIP runtime refused a launch */
 #define BSATTN_ERR_RANGE (-8)      /* a size exceeds what 32-bit indices can address */
+#define BSATTN_ERR_STATIC_LIMIT (-9) /* bsattn_fwd_static: the shape needs more scratch memory than
+                                        BSATTN_STATIC_SCRATCH_BYTES */
 
 /* dtype codes */
 #define BSATTN_F16 0
@@ -135,6 +137,25 @@ int bsattn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
                const int64_t* o_strides, void* workspace, size_t workspace_bytes,
                void* stream);
+
+/* Forward that allocates nothing and needs no workspace argument.  It has no counterpart in the
+ * reference; it is for callers that cannot allocate device memory around the call: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid allocation.  Same arguments, results and
+ * kernels as bsattn_fwd, with the workspace replaced by a device array of
+ * BSATTN_STATIC_SCRATCH_BYTES that is part of the library (every GPU the library runs on holds its
+ * own copy until the process ends).  Shapes whose bsattn_fwd_workspace exceeds that size are
+ * rejected with BSATTN_ERR_STATIC_LIMIT before any device work.  All calls on one GPU share the
+ * array: two calls that overlap in time on the same GPU (different streams or threads) race and
+ * must be serialised by the caller; calls on one stream are ordered and safe.  Nothing has to be
+ * cleared between calls (stale contents are told apart by a per-launch number).  The first call on
+ * a device looks up the array's address (no allocation, but not capturable: make one call before
+ * capturing). */
+#define BSATTN_STATIC_SCRATCH_BYTES (16u << 20)
+int bsattn_fwd_static(const void* q, const void* k, const void* v, void* o, float* lse,
+                      const int32_t* row_ptr, const int32_t* col_idx, int Bm, int Hm,
+                      int B, int H, int N, int D, int dtype, int out_dtype, float sm_scale,
+                      const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                      const int64_t* o_strides, void* stream);
 
 /* ------------------------------------------------------------------------------------
  * Forward with an elementwise mask: as bsattn_fwd, and inside the kept tiles flagged in

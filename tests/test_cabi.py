@@ -24,8 +24,8 @@ def test_strerror():
     from fa2_custom_mask import _ext
     l = _ext.lib()
     assert l.bsattn_strerror(0) == b"ok"
-    msgs = {l.bsattn_strerror(c) for c in range(-8, 1)}
-    assert len(msgs) == 9 and b"unknown error code" not in msgs
+    msgs = {l.bsattn_strerror(c) for c in range(-9, 1)}
+    assert len(msgs) == 10 and b"unknown error code" not in msgs
     assert l.bsattn_strerror(-99) == b"unknown error code"
 
 
