@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 LIB = os.path.join(HERE, "fa2_custom_mask", "libbsattn.so")
-SOURCES = ["api.hip", "mask_index.hip", "attn_fwd.hip", "attn_fwd_pair.hip", "attn_bwd.hip", "reorder.hip", "calibrate.hip"]
+SOURCES = ["api.hip", "mask_index.hip", "attn_fwd.hip", "attn_fwd_pair.hip", "attn_fwd_quad.hip", "attn_bwd.hip", "reorder.hip", "calibrate.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-I" + INCLUDE, "-I" + CSRC,
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",   # no packed fp32 VALU ops
          "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option"]

@@ -32,15 +32,6 @@
 
 namespace bsattn {
 
-// Partial results cross workgroups (and the L2 slices of different XCDs) inside one launch:
-// they are written and read with device-scope accesses, which go to the point of coherence.
-__device__ __forceinline__ void coherent_store(float* p, float v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ float coherent_load(const float* p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
 // A workgroup is four wavefronts, one per SIMD.  At D=64 a wavefront needs 256 registers and two
 // workgroups share a compute unit (while one merges or waits for its first tiles the other computes);
 // at D=128 a wavefront needs all 512 registers of its SIMD.
@@ -869,14 +860,24 @@ static size_t pair_parts_bytes(int B, int H, int N, int D, int split) {
   return split > 1 ? (size_t)split * B * H * N * (D + 2) * sizeof(float) : 0;
 }
 
-size_t fwd_workspace_bytes(int B, int H, int N, int D) {
+static int quad_slots_of_device() { return 2 * compute_units(); }   // two wavefront groups per workgroup, one workgroup per compute unit
+
+size_t coop_workspace_bytes(int B, int H, int N, int D) {
   if (D == 256) return 256 + pair_parts_bytes(B, H, N, D, pair_split(B, H, N / 64, D));   // the pair kernel only
   const int nb = N / 64;
   const int W = groups_per_head(B, H, nb, D);
   return slots_bytes(B, H, W, D) + (size_t)B * H * W * sizeof(unsigned long long);
 }
 
+// one size for bsattn_fwd, bsattn_fwd_elementwise and bsattn_fwd_quads
+size_t fwd_workspace_bytes(int B, int H, int N, int D) {
+  const size_t coop = coop_workspace_bytes(B, H, N, D);
+  const size_t quad = D == 64 ? quad_workspace_bytes(quad_slots_of_device(), B, H, N / 64) : 0;
+  return coop > quad ? coop : quad;
+}
+
 void launch_fwd_pair(const FwdParams& prm, int D, int dt, bool elementwise, hipStream_t st);   // attn_fwd_pair.hip
+void launch_fwd_quad(const FwdParams& prm, int dt, hipStream_t st);                            // attn_fwd_quad.hip
 // D = 128 with enough row blocks in the launch to fill the chip goes to the kernel that gives each
 // row block to one wavefront pair (two wavefronts per SIMD, no merges between workgroups).  With
 // fewer row blocks its critical path is the longest row, which the host cannot see (the lists
@@ -977,6 +978,25 @@ int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
     if (s.D == 64) { if (dt == 0) launch_fwd_t<64, 0, true>(prm, BH, st); else if (dt == 1) launch_fwd_t<64, 1, true>(prm, BH, st); else launch_fwd_t<64, 2, true>(prm, BH, st); }
     else { if (dt == 0) launch_fwd_t<128, 0, true>(prm, BH, st); else if (dt == 1) launch_fwd_t<128, 1, true>(prm, BH, st); else launch_fwd_t<128, 2, true>(prm, BH, st); }
   }
+  return launch_status();
+}
+
+// Forward over quad lists (attn_fwd_quad.hip): head dimension 64, block masks.
+int launch_fwd_quads(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* row_ptr,
+                     const int32_t* quad_ptr, const int32_t* quad_list, const AttnShape& s, void* ws, hipStream_t st) {
+  FwdParams prm = {};
+  prm.q = q; prm.k = k; prm.v = v; prm.o = o; prm.lse = lse;
+  prm.row_ptr = row_ptr; prm.quad_ptr = quad_ptr; prm.quad_list = quad_list; prm.ws = (float*)ws;
+  prm.B = s.B; prm.H = s.H; prm.N = s.N; prm.nb = s.N / 64; prm.Bm = s.Bm; prm.Hm = s.Hm;
+  prm.epoch = next_epoch();
+  prm.out_f32 = s.out_dtype == BSATTN_F32;
+  prm.qk_scale = s.sm_scale * 1.4426950408889634f;
+  for (int i = 0; i < 3; ++i) { prm.qs[i] = s.qs[i]; prm.ks[i] = s.ks[i]; prm.vs[i] = s.vs[i]; prm.os[i] = s.os[i]; }
+  prm.qslots = quad_slots_of_device();
+  prm.qcounters = (unsigned long long*)((char*)ws + quad_parts_bytes(prm.qslots));
+  prm.vt = (const unsigned short*)((char*)prm.qcounters + quad_counters_bytes(s.B, s.H, prm.nb));
+  const bool bf = s.dtype == BSATTN_BF16;
+  launch_fwd_quad(prm, !bf ? 0 : (prm.out_f32 ? 1 : 2), st);
   return launch_status();
 }
 

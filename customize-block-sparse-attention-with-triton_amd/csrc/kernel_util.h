@@ -156,6 +156,15 @@ __device__ __forceinline__ void store_out4(void* obase, int64_t elem_off, bool o
 }
 
 
+// Partial results cross workgroups (and the L2 slices of different XCDs) inside one launch:
+// they are written and read with device-scope accesses, which go to the point of coherence.
+__device__ __forceinline__ void coherent_store(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float coherent_load(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // Swizzle for tiles that are read both ways (operand reads of 32 consecutive rows and
 // transpose reads of 4 consecutive rows x 64 bytes): a bijection of the row bits that
 // separates both access patterns over the 64 LDS banks.

@@ -29,6 +29,9 @@ _SIGNATURES = {
     "bsattn_fwd_workspace": ([_i, _i, _i, _i, ctypes.POINTER(ctypes.c_size_t)], _i),
     "bsattn_fwd": ([_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f,
                     _p, _p, _p, _p, _p, ctypes.c_size_t, _p], _i),
+    "bsattn_quad_lists": ([_p, _p, _i, _i, _i, _p, _p, _p, _p], _i),
+    "bsattn_fwd_quads": ([_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f,
+                          _p, _p, _p, _p, _p, ctypes.c_size_t, _p], _i),
     "bsattn_fwd_static": ([_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f,
                            _p, _p, _p, _p, _p], _i),
     "bsattn_fwd_elementwise": ([_p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f,

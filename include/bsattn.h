@@ -85,6 +85,22 @@ int bsattn_block_mask_to_lists(const uint8_t* block, int Bm, int Hm, int nb,
                                int32_t* counts, void* workspace, size_t workspace_bytes,
                                void* stream);
 
+/* Quad lists: a second form of the kept-tile lists, for bsattn_fwd_quads.  Four consecutive row
+ * blocks of a mask head form a quad (the last quad of a head may hold fewer).  For quad j
+ * (j = mask head * ceil(nb/4) + index within the head):
+ *   quad_list[j*nb + i], i < size_j: the i-th column block, ascending, that any row block of the quad
+ *       keeps, in bits 0..15, and in bits 16..19 which of the quad's row blocks keep it;
+ *   quad_ptr  int32 [Bm*Hm*ceil(nb/4) + 1]: exclusive prefix sums of size_j;
+ *   quad_stats int32 [2]: sum of all size_j, and the number of kept tiles of the mask.  Walking the
+ *       unions costs 4 * quad_stats[0] tile slots for quad_stats[1] kept tiles: the closer the
+ *       ratio quad_stats[1] / (4 * quad_stats[0]) is to 1, the better bsattn_fwd_quads does.
+ * row_ptr / col_idx as made by bsattn_block_mask_to_lists for the same [Bm,Hm,nb,nb] mask;
+ * quad_list has capacity Bm*Hm*ceil(nb/4)*nb; nb <= BSATTN_QUAD_MAX_BLOCKS.  No counterpart in the
+ * reference, whose kernel walks one row list per program (fa2_custom_mask/fa2_fwd.py:152-153). */
+#define BSATTN_QUAD_MAX_BLOCKS 2048
+int bsattn_quad_lists(const int32_t* row_ptr, const int32_t* col_idx, int Bm, int Hm, int nb,
+                      int32_t* quad_ptr, int32_t* quad_list, int32_t* quad_stats, void* stream);
+
 /* ------------------------------------------------------------------------------------
  * Elementwise masks (exact semantics inside partly set tiles: the naive masked_fill(-inf)
  * of kernel-test.py:38, which the reference's dead elementwise loop fa2_fwd.py:67-73 and
@@ -138,12 +154,31 @@ int bsattn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                const int64_t* o_strides, void* workspace, size_t workspace_bytes,
                void* stream);
 
+/* The same forward (same arguments, same results up to rounding) by a kernel made for masks whose
+ * neighbouring row blocks keep nearly the same column blocks: dense, block-causal, banded, frame-wise
+ * masks.  The four row blocks of a quad walk the union of their column lists together and share
+ * every K and V tile, so a launch computes on 4 * quad_stats[0] tile slots instead of
+ * quad_stats[1] tiles (see bsattn_quad_lists): at a ratio near 1 it is the faster entry point, for
+ * scattered masks bsattn_fwd is.  Replaces the same reference launch as bsattn_fwd
+ * (fa2_custom_mask/fa2_custom_mask.py:69-87).  Head dimension 64 only (BSATTN_ERR_HEAD_DIM);
+ * N <= 64 * BSATTN_QUAD_MAX_BLOCKS, (Bm, Hm) = (1, 1) or (B, H), and at most 4096 quads in the
+ * launch (per head for a shared mask): BSATTN_ERR_RANGE otherwise.  Workspace as bsattn_fwd
+ * (bsattn_fwd_workspace bytes).  Row blocks shared between workgroups are finished by the
+ * workgroup that arrives last (a counter per row block in the workspace, no waiting). */
+int bsattn_fwd_quads(const void* q, const void* k, const void* v, void* o, float* lse,
+                     const int32_t* row_ptr, const int32_t* quad_ptr, const int32_t* quad_list,
+                     int Bm, int Hm, int B, int H, int N, int D, int dtype, int out_dtype,
+                     float sm_scale, const int64_t* q_strides, const int64_t* k_strides,
+                     const int64_t* v_strides, const int64_t* o_strides, void* workspace,
+                     size_t workspace_bytes, void* stream);
+
 /* Forward that allocates nothing and needs no workspace argument.  It has no counterpart in the
  * reference; it is for callers that cannot allocate device memory around the call: code under HIP
  * graph capture, tight serving loops, harnesses that forbid allocation.  Same arguments, results and
  * kernels as bsattn_fwd, with the workspace replaced by a device array of
  * BSATTN_STATIC_SCRATCH_BYTES that is part of the library (every GPU the library runs on holds its
- * own copy until the process ends).  Shapes whose bsattn_fwd_workspace exceeds that size are
+ * own copy until the process ends).  Shapes whose parts and flags (the memory
+ * bsattn_fwd's kernels use out of its workspace) exceed that size are
  * rejected with BSATTN_ERR_STATIC_LIMIT before any device work.  All calls on one GPU share the
  * array: two calls that overlap in time on the same GPU (different streams or threads) race and
  * must be serialised by the caller; calls on one stream are ordered and safe.  Nothing has to be

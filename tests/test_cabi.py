@@ -93,3 +93,18 @@ def test_python_wrapper_rejects_bad_input_without_gpu():
         fm.build_groups_from_block_mask(torch.ones(1, 1, 2, 2))
     with pytest.raises(RuntimeError):
         fm.build_groups_from_block_mask(m)                                       # CPU mask: no CPU path
+
+
+def test_quad_split_arithmetic(tmp_path):
+    """The work split of the forward kernel that walks quads (csrc/fwd_quad_split.h) is plain integer
+    arithmetic shared with the kernel: a host program checks on random weight axes that the ranges
+    tile the axis and that every quad's parts are the ranges quad_parts() names (built with the
+    address and undefined-behaviour sanitizers)."""
+    import subprocess
+    exe = str(tmp_path / "quad_split_check")
+    src = os.path.join(ROOT, "tests", "quad_split_check.cpp")
+    inc = os.path.join(ROOT, "customize-block-sparse-attention-with-triton_amd", "csrc")
+    subprocess.run(["g++", "-O1", "-std=c++17", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
+                    "-static-libasan", "-I" + inc, src, "-o", exe], check=True)
+    out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout
+    assert out.startswith("ok ")
