@@ -9,6 +9,8 @@ extern "C" {
 
 int bsattn_version(void) { return BSATTN_VERSION; }
 
+int bsattn_set_deterministic(int on) { return set_deterministic(on); }
+
 const char* bsattn_strerror(int code) {
   switch (code) {
     case BSATTN_OK: return "ok";

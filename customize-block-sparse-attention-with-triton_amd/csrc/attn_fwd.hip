@@ -605,7 +605,8 @@ void fwd_kernel(const FwdParams prm) {
           const bool has1 = nxt < seg_b, copy_v = has1;
           int nn = 0, cb_nn_v = 0;
           tile(has1, cb_nxt & COL_MASK, nxt, copy_v, (cx >> 30) != 0, [&] {
-            nn = __builtin_amdgcn_readfirstlane(drawn);
+            // (deterministic: every wavefront takes every NW-th tile, whatever its pace)
+            nn = prm.deterministic ? nxt + NW : __builtin_amdgcn_readfirstlane(drawn);
             cb_nn_v = nn < g1 ? col_of(nn) : 0;     // looked up now, needed at the end of the tile
           });
           if (has1) kdone = nxt;
@@ -633,21 +634,26 @@ void fwd_kernel(const FwdParams prm) {
             ml[(w * 2 + 1) * 64 + qb * 32 + ln] = mass ? lsum[qb] : 0.f;
           }
         }
-        // A row block cut by range boundaries is finished by the workgroup that holds its first
-        // tiles (for that workgroup it is the last row block of its range): the other workgroups
-        // publish their parts (for them it is the first row block of their ranges, so the parts
-        // are ready early), and the finishing workgroup pulls them.
+        // A row block cut by range boundaries has one part per workgroup that holds tiles of it.  Every
+        // such workgroup publishes its part and then counts itself in; the one that finds all the
+        // others counted merges the parts and writes the row block.  Nobody waits for anybody, so
+        // the result does not depend on which workgroups are resident at the same time.
         const bool has_head = seg_a == row_s, has_tail = seg_b == row_e;
-        const bool full = has_head && has_tail, publish = !has_head, pull = has_head && !has_tail;
+        const bool full = has_head && has_tail;
         float wgt[NW][2];   // weight of wavefront p's partial for this lane's query of block qb
         float M[2], L[2];
-        float keep[C::ROUNDS][C::QPW][4];   // this wavefront's share of the merged accumulator (pull)
+        float keep[C::ROUNDS][C::QPW][4];   // this wavefront's share of the workgroup's part
         // A zero the compiler cannot see through (ctr[3] stays 0): the per-lane addresses into the
         // workspace do not change from row block to row block and would otherwise be computed
         // once, up front, and occupy registers throughout the tile loops.
         typedef volatile int __attribute__((address_space(3)))* lds_vint_ptr_t;
         const int zero = *(lds_vint_ptr_t)(lds_ptr_t)(ctr + 3);
-        float* slot = prm.ws + ((int64_t)bh * prm.W + wg) * partial_floats(D) + zero;
+        // two slots per workgroup: a range can end inside one row block (that part goes to slot 1: it
+        // holds the row block's first tiles) after having begun inside another (slot 0)
+        auto slot_of = [&](int p, bool head) {
+          return prm.ws + (((int64_t)bh * prm.W + p) * 2 + (head ? 1 : 0)) * partial_floats(D) + zero;
+        };
+        float* slot = slot_of(wg, has_head);
 #pragma unroll
         for (int rd = 0; rd < C::ROUNDS; ++rd) {
           {
@@ -695,7 +701,7 @@ void fwd_kernel(const FwdParams prm) {
               const int64_t qrow = (int64_t)(r * 64 + qb * 32 + ln);
               store_out4<BF16>(obase, qrow * prm.os[2] + 32 * db + 8 * i4 + 4 * g, prm.out_f32, x[0] * inv, x[1] * inv,
                                x[2] * inv, x[3] * inv);
-            } else if (publish) {
+            } else {
 #pragma unroll
               for (int e = 0; e < 4; ++e) coherent_store(slot + (idx0 + e) * 64 + lane, x[e]);
             }
@@ -711,7 +717,7 @@ void fwd_kernel(const FwdParams prm) {
               prm.lse[((int64_t)bh * prm.N) + (int64_t)(r * 64 + qb * 32 + ln)] =
                   L[qb] > 0.f ? (M[qb] + __builtin_amdgcn_logf(L[qb])) * 0.6931471805599453f : -INFINITY;
           }
-        } else if (publish) {
+        } else {
           if (w == 0 && g == 0) {
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb) {
@@ -719,87 +725,113 @@ void fwd_kernel(const FwdParams prm) {
               coherent_store(slot + 64 * D + 64 + qb * 32 + ln, L[qb]);
             }
           }
-          // the flag goes up once every wavefront's stores have been acknowledged
+          // The workgroups pf .. pl hold the parts of this row block: pf is the one before the first range
+          // boundary that stays inside the row block (boundaries close to an end move there), pl the one
+          // after the last.  Every holder computes the same two numbers.
+          int pl_ = split_of_tile(hs, row_e - 1), pf_ = split_of_tile(hs, row_s);
+          while (pl_ > pf_ && snap_boundary<C::SNAP>(split_begin(hs, pl_), row_s, row_e) >= row_e) --pl_;
+          while (pf_ < pl_ && snap_boundary<C::SNAP>(split_begin(hs, pf_ + 1), row_s, row_e) <= row_s) ++pf_;
+          const int nparts = pl_ - pf_ + 1;
+          // The part is counted in once every wavefront's stores have been acknowledged (vmcnt 0, then the
+          // barrier).  Every access to a part, stores here and loads below, is itself an access at device
+          // scope: it is served by the memory all compute units share, never by a cache that only
+          // some of them see.  The counter update is therefore relaxed: release / acquire order on it
+          // would add a write-back and an invalidation of this die's whole L2, measured at 9 us per
+          // launch (keep 0.1, N = 17536: 31 -> 41 us), to order accesses that are already ordered.
+          // The counter holds (launch mark << 16 | parts counted); stale contents carry another mark.
           wait_vm<0>();
           __syncthreads();
-          if (threadIdx.x == 0)
-            __hip_atomic_store(prm.flags + (int64_t)bh * prm.W + wg, prm.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        } else {
-          // pull the parts of the workgroups wg+1 .. pl and finish the row block
-          // (the last workgroup with tiles of this row block: a later one whose start moved to the row
-          // block's end holds none)
-          int pl_ = split_of_tile(hs, row_e - 1);
-          while (pl_ > wg && snap_boundary<C::SNAP>(split_begin(hs, pl_), row_s, row_e) >= row_e) --pl_;
-          bool ok = true;
-          for (int p = wg + 1; p <= pl_; ++p) {
-            unsigned long long* fl = prm.flags + (int64_t)bh * prm.W + p;
-            // The wait is bounded (about 0.2 s of the 100 MHz counter): a part that never arrives
-            // turns the row block into NaNs instead of a hang.
-            const long long t_start = __builtin_amdgcn_s_memrealtime();
-            while (__hip_atomic_load(fl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != prm.epoch) {
-              if (__builtin_amdgcn_s_memrealtime() - t_start > 20000000ll) { ok = false; break; }
-              __builtin_amdgcn_s_sleep(4);
+          unsigned long long* arrivals = prm.flags + (int64_t)bh * nb + r;
+          if (threadIdx.x == 0) {
+            unsigned long long old = __hip_atomic_load(arrivals, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (;;) {     // (ends: the counter only changes when another part is counted, at most nparts times)
+              const unsigned long long want = (old >> 16) == prm.epoch ? old + 1 : ((prm.epoch << 16) | 1ull);
+              if (__hip_atomic_compare_exchange_strong(arrivals, &old, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_AGENT)) {
+                ctr[4] = (int)(want & 0xffffull);
+                break;
+              }
             }
-            const float* sp = prm.ws + ((int64_t)bh * prm.W + p) * partial_floats(D) + zero;
-            // all loads of the part are issued before the first one is waited for (a round trip
-            // to the point of coherence costs about a microsecond)
-            float mp[2], lp[2], dat[C::ROUNDS][C::QPW][4];
-#pragma unroll
-            for (int qb = 0; qb < 2; ++qb) {
-              mp[qb] = coherent_load(sp + 64 * D + qb * 32 + ln);
-              lp[qb] = coherent_load(sp + 64 * D + 64 + qb * 32 + ln);
-            }
+          }
+          __syncthreads();
+          const int counted = __builtin_amdgcn_readfirstlane(*(lds_vint_ptr_t)(lds_ptr_t)(ctr + 4));
+          if (counted == nparts) {
+            // last one in: every part is in memory.  They are summed in the order of the ranges, whoever
+            // does it, so the result does not depend on the order of arrival.
+            float Ms[2] = {-INFINITY, -INFINITY}, Ls[2] = {0.f, 0.f}, acc[C::ROUNDS][C::QPW][4];
 #pragma unroll
             for (int rd = 0; rd < C::ROUNDS; ++rd)
 #pragma unroll
               for (int tq = 0; tq < C::QPW; ++tq)
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                  dat[rd][tq][e] = coherent_load(sp + (rd * C::R + 4 * (w * C::QPW + tq) + e) * 64 + lane);
-            __builtin_amdgcn_sched_barrier(0);
-            float sc_own[2], sc_p[2];
+                for (int e = 0; e < 4; ++e) acc[rd][tq][e] = 0.f;
+            for (int p = pf_; p <= pl_; ++p) {
+              float mp[2], lp[2], dat[C::ROUNDS][C::QPW][4];
+              if (p == wg) {
 #pragma unroll
-            for (int qb = 0; qb < 2; ++qb) {
-              const float mn = fmaxf(M[qb], mp[qb]);     // a side without mass has maximum -inf and weight 0
-              sc_own[qb] = M[qb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(M[qb] - mn);
-              sc_p[qb] = mp[qb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mp[qb] - mn);
-              L[qb] = L[qb] * sc_own[qb] + lp[qb] * sc_p[qb];
-              M[qb] = mn;
+                for (int qb = 0; qb < 2; ++qb) { mp[qb] = M[qb]; lp[qb] = L[qb]; }
+#pragma unroll
+                for (int rd = 0; rd < C::ROUNDS; ++rd)
+#pragma unroll
+                  for (int tq = 0; tq < C::QPW; ++tq)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) dat[rd][tq][e] = keep[rd][tq][e];
+              } else {
+                const float* sp = slot_of(p, p == pf_);
+                // all loads of the part are issued before the first one is waited for (a round trip
+                // to the point of coherence costs about a microsecond)
+#pragma unroll
+                for (int qb = 0; qb < 2; ++qb) {
+                  mp[qb] = coherent_load(sp + 64 * D + qb * 32 + ln);
+                  lp[qb] = coherent_load(sp + 64 * D + 64 + qb * 32 + ln);
+                }
+#pragma unroll
+                for (int rd = 0; rd < C::ROUNDS; ++rd)
+#pragma unroll
+                  for (int tq = 0; tq < C::QPW; ++tq)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                      dat[rd][tq][e] = coherent_load(sp + (rd * C::R + 4 * (w * C::QPW + tq) + e) * 64 + lane);
+                __builtin_amdgcn_sched_barrier(0);
+              }
+              float sc_own[2], sc_p[2];
+#pragma unroll
+              for (int qb = 0; qb < 2; ++qb) {
+                const float mn = fmaxf(Ms[qb], mp[qb]);     // a side without mass has maximum -inf and weight 0
+                sc_own[qb] = Ms[qb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(Ms[qb] - mn);
+                sc_p[qb] = mp[qb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mp[qb] - mn);
+                Ls[qb] = Ls[qb] * sc_own[qb] + lp[qb] * sc_p[qb];
+                Ms[qb] = mn;
+              }
+#pragma unroll
+              for (int rd = 0; rd < C::ROUNDS; ++rd)
+#pragma unroll
+                for (int tq = 0; tq < C::QPW; ++tq) {
+                  const int qb = ((rd * C::R + 4 * (w * C::QPW + tq)) / 16) & 1;
+#pragma unroll
+                  for (int e = 0; e < 4; ++e) acc[rd][tq][e] = acc[rd][tq][e] * sc_own[qb] + sc_p[qb] * dat[rd][tq][e];
+                }
             }
 #pragma unroll
             for (int rd = 0; rd < C::ROUNDS; ++rd)
 #pragma unroll
               for (int tq = 0; tq < C::QPW; ++tq) {
-                const int qb = ((rd * C::R + 4 * (w * C::QPW + tq)) / 16) & 1;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) keep[rd][tq][e] = keep[rd][tq][e] * sc_own[qb] + sc_p[qb] * dat[rd][tq][e];
+                const int idx0 = rd * C::R + 4 * (w * C::QPW + tq);
+                const int db = idx0 / 32, qb = (idx0 / 16) & 1, i4 = (idx0 & 15) / 4;
+                const float inv = Ls[qb] > 0.f ? 1.0f / Ls[qb] : 0.f;
+                const int64_t qrow = (int64_t)(r * 64 + qb * 32 + ln);
+                store_out4<BF16>(obase, qrow * prm.os[2] + 32 * db + 8 * i4 + 4 * g, prm.out_f32,
+                                 acc[rd][tq][0] * inv, acc[rd][tq][1] * inv, acc[rd][tq][2] * inv, acc[rd][tq][3] * inv);
               }
-          }
-          const float bad = ok ? 0.f : __builtin_nanf("");
+            if (w == 0 && g == 0 && prm.lse != nullptr) {
 #pragma unroll
-          for (int rd = 0; rd < C::ROUNDS; ++rd)
-#pragma unroll
-            for (int tq = 0; tq < C::QPW; ++tq) {
-              const int idx0 = rd * C::R + 4 * (w * C::QPW + tq);
-              const int db = idx0 / 32, qb = (idx0 / 16) & 1, i4 = (idx0 & 15) / 4;
-              const float inv = L[qb] > 0.f ? 1.0f / L[qb] : 0.f;
-              const int64_t qrow = (int64_t)(r * 64 + qb * 32 + ln);
-              store_out4<BF16>(obase, qrow * prm.os[2] + 32 * db + 8 * i4 + 4 * g, prm.out_f32,
-                               keep[rd][tq][0] * inv + bad, keep[rd][tq][1] * inv + bad, keep[rd][tq][2] * inv + bad,
-                               keep[rd][tq][3] * inv + bad);
+              for (int qb = 0; qb < 2; ++qb)
+                prm.lse[((int64_t)bh * prm.N) + (int64_t)(r * 64 + qb * 32 + ln)] =
+                    Ls[qb] > 0.f ? (Ms[qb] + __builtin_amdgcn_logf(Ls[qb])) * 0.6931471805599453f : -INFINITY;
             }
-          if (w == 0 && g == 0 && prm.lse != nullptr) {
-#pragma unroll
-            for (int qb = 0; qb < 2; ++qb)
-              prm.lse[((int64_t)bh * prm.N) + (int64_t)(r * 64 + qb * 32 + ln)] =
-                  (L[qb] > 0.f ? (M[qb] + __builtin_amdgcn_logf(L[qb])) * 0.6931471805599453f : -INFINITY) + bad;
+            // back to zero, so that a replay of this launch (same mark) starts from a clean counter
+            if (threadIdx.x == 0) __hip_atomic_store(arrivals, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
-          // every wavefront has read the flags: put them back to zero, so that a replay of this
-          // launch (same epoch) does not take this launch's parts for its own
-          __syncthreads();
-          if (threadIdx.x == 0)
-            for (int p = wg + 1; p <= pl_; ++p)
-              __hip_atomic_store(prm.flags + (int64_t)bh * prm.W + p, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
       }
       t = seg_b;
@@ -817,6 +849,11 @@ static unsigned long long next_epoch() {
   do { e = counter.fetch_add(1) & 0xffffffffffffull; } while (e == 0);
   return e;
 }
+
+// Process-wide switch: results that do not depend on the pace of the wavefronts (bsattn_set_deterministic).
+static std::atomic<int> deterministic_mode{0};
+int set_deterministic(int on) { return deterministic_mode.exchange(on != 0 ? 1 : 0); }
+int get_deterministic() { return deterministic_mode.load(); }
 
 int compute_units() {
   static int cached[64] = {0};   // per device; the value never changes, so a race only repeats the query
@@ -839,9 +876,9 @@ static int groups_per_head(int B, int H, int nb, int D) {
   return (int)W;
 }
 
-// workspace: partial slots [B*H][W][partial_floats] (fp32), then their flags [B*H][W] (64 bit)
+// workspace: partial slots [B*H][W][2][partial_floats] (fp32), then the arrival counters [B*H][nb] (64 bit)
 static size_t slots_bytes(int B, int H, int W, int D) {
-  return (size_t)B * H * W * partial_floats(D) * sizeof(float);
+  return (size_t)B * H * W * 2 * partial_floats(D) * sizeof(float);
 }
 
 // Pair kernel: workgroups per row block.  One when the launch has enough row blocks to fill the GPU twice
@@ -866,7 +903,7 @@ size_t coop_workspace_bytes(int B, int H, int N, int D) {
   if (D == 256) return 256 + pair_parts_bytes(B, H, N, D, pair_split(B, H, N / 64, D));   // the pair kernel only
   const int nb = N / 64;
   const int W = groups_per_head(B, H, nb, D);
-  return slots_bytes(B, H, W, D) + (size_t)B * H * W * sizeof(unsigned long long);
+  return slots_bytes(B, H, W, D) + (size_t)B * H * nb * sizeof(unsigned long long);
 }
 
 // one size for bsattn_fwd, bsattn_fwd_elementwise and bsattn_fwd_quads
@@ -952,6 +989,7 @@ int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
   prm.first_ids = (s.D == 64 ? FwdCfg<64>::WG_PER_CU : FwdCfg<128>::WG_PER_CU) > 1 ? compute_units() : 0;
   prm.flags = (unsigned long long*)((char*)ws + slots_bytes(s.B, s.H, prm.W, s.D));
   prm.epoch = next_epoch();
+  prm.deterministic = get_deterministic();
   prm.out_f32 = s.out_dtype == BSATTN_F32;
   prm.qk_scale = s.sm_scale * 1.4426950408889634f;
   for (int i = 0; i < 3; ++i) { prm.qs[i] = s.qs[i]; prm.ks[i] = s.ks[i]; prm.vs[i] = s.vs[i]; prm.os[i] = s.os[i]; }

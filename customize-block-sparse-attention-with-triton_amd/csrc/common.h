@@ -47,6 +47,8 @@ inline void once_per_device(std::atomic<unsigned long long>& done, F&& f) {
   done.fetch_or(bit, std::memory_order_release);
 }
 size_t fwd_workspace_bytes(int B, int H, int N, int D);
+int set_deterministic(int on);   // returns the previous setting
+int get_deterministic();
 int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                const int32_t* row_ptr, const int32_t* col_idx, const uint8_t* tile_partial,
                const uint64_t* tile_bits, const AttnShape& s, void* ws, hipStream_t st);

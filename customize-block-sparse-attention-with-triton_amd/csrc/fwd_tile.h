@@ -11,9 +11,10 @@ struct FwdParams {
   const int32_t* row_ptr; const int32_t* col_idx;
   const unsigned char* tile_partial;        // elementwise masks: per kept tile, 1 = only partly set
   const unsigned long long* tile_bits;      // ... and its 64 row words (bit c = column c)
-  float* ws;                       // partial slots of row blocks shared between workgroups
-  unsigned long long* flags;       // one per slot: holds `epoch` once the slot's part is complete
-  unsigned long long epoch;        // distinguishes this launch's flags from stale contents
+  float* ws;                       // partial slots of row blocks shared between workgroups (two per workgroup)
+  unsigned long long* flags;       // one per row block: parts counted in so far, tagged with `epoch`
+  unsigned long long epoch;        // distinguishes this launch's counters from stale contents
+  int deterministic;               // tiles go to the wavefronts of a workgroup in a fixed pattern
   int split;                       // pair kernel: workgroups per row block (1: results written directly)
   float* part_o; float* part_ml;   // split > 1: unnormalised fp32 O parts [split][B*H][N][D] and their (m, l) [split][B*H][N][2]
   int B, H, N, nb, Bm, Hm, W;   // W: workgroups per head

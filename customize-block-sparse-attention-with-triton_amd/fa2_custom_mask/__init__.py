@@ -4,7 +4,7 @@ Exports the names of the reference package (fa2_custom_mask/__init__.py:1-5) exc
 Triton kernel objects, which have no counterpart here."""
 from .fa2_custom_mask import (flash_attention_custom_mask, flash_attention_custom_mask_lse,
                               attention_forward_backward, build_groups_from_block_mask, _attention,
-                              ForwardPlan, BackwardPlan)
+                              ForwardPlan, BackwardPlan, set_deterministic)
 from .utils import is_hip, keep, reduce_dense_mask, block_mask_to_lists, TileLists
 from .functional import (permute_qkv_triton, apply_head_wise_reorder, inv_permute_attn_triton,
                          apply_inv_reorder)
@@ -12,6 +12,6 @@ from .functional import (permute_qkv_triton, apply_head_wise_reorder, inv_permut
 __all__ = [
     "flash_attention_custom_mask", "flash_attention_custom_mask_lse", "attention_forward_backward",
     "build_groups_from_block_mask", "is_hip", "keep", "reduce_dense_mask", "block_mask_to_lists",
-    "TileLists", "ForwardPlan", "BackwardPlan", "permute_qkv_triton", "apply_head_wise_reorder", "inv_permute_attn_triton",
+    "TileLists", "ForwardPlan", "BackwardPlan", "set_deterministic", "permute_qkv_triton", "apply_head_wise_reorder", "inv_permute_attn_triton",
     "apply_inv_reorder",
 ]

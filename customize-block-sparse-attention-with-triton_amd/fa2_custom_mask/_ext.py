@@ -19,6 +19,7 @@ _DTYPE_CODE = {torch.float16: F16, torch.bfloat16: BF16, torch.float32: F32}
 _i, _i64, _p, _f = ctypes.c_int, ctypes.c_int64, ctypes.c_void_p, ctypes.c_float
 _SIGNATURES = {
     "bsattn_version": ([], _i),
+    "bsattn_set_deterministic": ([_i], _i),
     "bsattn_strerror": ([_i], ctypes.c_char_p),
     "bsattn_reduce_dense_mask": ([_p, _i, _i, _i, _i64, _i64, _i64, _p, _p], _i),
     "bsattn_mask_lists_workspace": ([_i, _i, _i, ctypes.POINTER(ctypes.c_size_t)], _i),

@@ -79,6 +79,14 @@ def _dense_mask(device, nb):
     return _all_true[key]
 
 
+def set_deterministic(on):
+    """Process-wide switch (bsattn_set_deterministic), returns the previous setting.  On: two runs of the
+    forward on the same inputs give the same bits; off (the default): the tiles of a row block go to
+    the wavefronts as they become free, which is faster and changes the last bits from run to run.
+    The backward is deterministic either way."""
+    return bool(_ext.lib().bsattn_set_deterministic(1 if on else 0))
+
+
 QUAD_MIN_EFFICIENCY = 0.7
 # The kernel that walks quads is chosen by the caller (ForwardPlan(quads=True), or this switch for the
 # autograd path): at the sizes measured so far the kernel behind bsattn_fwd is the faster of the two.

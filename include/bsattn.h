@@ -49,6 +49,13 @@ extern "C" {
 #define BSATTN_F32 2 /* outputs only */
 
 int bsattn_version(void);
+/* Process-wide switch (default off), returns the previous setting.  On: the forward's result
+ * depends on nothing but its inputs and the device (two runs give the same bits).  Off: the
+ * tiles of a row block are handed to the wavefronts of a workgroup as they become free, which
+ * is faster and changes the order of summation, i.e. the last bits, from run to run.  The
+ * backward and the preprocessing are deterministic either way.  No counterpart in the
+ * reference (Triton's kernels there are deterministic by construction). */
+int bsattn_set_deterministic(int on);
 /* Static string for an error code; never freed by the caller. */
 const char* bsattn_strerror(int code);
 
@@ -146,7 +153,13 @@ int bsattn_fwd_workspace(int B, int H, int N, int D, size_t* bytes);
  * row_ptr/col_idx: lists from bsattn_block_mask_to_lists for a [Bm,Hm,nb,nb] mask,
  *        Bm in {1,B}, Hm in {1,H} (1 = shared across that axis).
  * Row blocks without a kept tile get O = 0 and lse = -inf (the reference leaves them
- * unwritten: fa2_custom_mask.py:29-30,59). */
+ * unwritten: fa2_custom_mask.py:29-30,59).
+ * A row block whose kept tiles are split over several workgroups is finished by the workgroup
+ * that completes its share last (parts and one counter per row block live in the workspace):
+ * no workgroup ever waits for another, so the call completes whatever else runs on the GPU
+ * and however many workgroups are resident at a time.  The workspace needs no initialisation
+ * and may be reused by the next call on the same stream; two calls that overlap in time need
+ * two workspaces. */
 int bsattn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                const int32_t* row_ptr, const int32_t* col_idx, int Bm, int Hm,
                int B, int H, int N, int D, int dtype, int out_dtype, float sm_scale,
@@ -185,7 +198,7 @@ int bsattn_fwd_quads(const void* q, const void* k, const void* v, void* o, float
  * cleared between calls (stale contents are told apart by a per-launch number).  The first call on
  * a device looks up the array's address (no allocation, but not capturable: make one call before
  * capturing). */
-#define BSATTN_STATIC_SCRATCH_BYTES (16u << 20)
+#define BSATTN_STATIC_SCRATCH_BYTES (32u << 20)
 int bsattn_fwd_static(const void* q, const void* k, const void* v, void* o, float* lse,
                       const int32_t* row_ptr, const int32_t* col_idx, int Bm, int Hm,
                       int B, int H, int N, int D, int dtype, int out_dtype, float sm_scale,

@@ -68,7 +68,7 @@ def test_static_forward_rejects_shapes_beyond_its_scratch(dev):
     n = ctypes.c_size_t()
     B, H, N, D = 1, 1, 17536, 256        # row lists shared between workgroups: fp32 parts of over 100 MB
     assert lib.bsattn_fwd_workspace(B, H, N, D, ctypes.byref(n)) == 0
-    if n.value <= (16 << 20):
+    if n.value <= (32 << 20):
         pytest.skip("this shape fits the static scratch on this device")
     P = ctypes.c_void_p(4096)             # never dereferenced: the size check comes first
     s = (ctypes.c_int64 * 4)(H * N * D, N * D, D, 1)
