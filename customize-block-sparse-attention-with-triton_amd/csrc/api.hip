@@ -222,7 +222,8 @@ static int bwd_common(const void* q, const void* k, const void* v, const void* o
                       const uint64_t* bits_rows, const uint64_t* bits_cols, int Bm, int Hm,
                       int B, int H, int N, int D, int dtype, int out_dtype, float sm_scale,
                       const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
-                      const int64_t* o_strides, const int64_t* do_strides, void* workspace,
+                      const int64_t* o_strides, const int64_t* do_strides, const int64_t* dq_strides,
+                      const int64_t* dk_strides, const int64_t* dv_strides, void* workspace,
                       size_t workspace_bytes, void* stream) {
   if (q == nullptr || k == nullptr || v == nullptr || o == nullptr || d_o == nullptr || lse == nullptr ||
       dq == nullptr || dk == nullptr || dv == nullptr || row_ptr == nullptr || col_idx == nullptr ||
@@ -235,11 +236,21 @@ static int bwd_common(const void* q, const void* k, const void* v, const void* o
   if ((rc = check_strides(v_strides, 2, v)) != BSATTN_OK) return rc;
   if ((rc = check_strides(o_strides, 2, o)) != BSATTN_OK) return rc;
   if ((rc = check_strides(do_strides, 2, d_o)) != BSATTN_OK) return rc;
+  // results: NULL strides mean [B, H, N, D] without gaps
+  const int64_t dense[4] = {(int64_t)H * N * D, (int64_t)N * D, D, 1};
+  const int out_bytes = out_dtype == BSATTN_F32 ? 4 : 2;
+  if (dq_strides == nullptr) dq_strides = dense;
+  if (dk_strides == nullptr) dk_strides = dense;
+  if (dv_strides == nullptr) dv_strides = dense;
+  if ((rc = check_strides(dq_strides, out_bytes, dq)) != BSATTN_OK) return rc;
+  if ((rc = check_strides(dk_strides, out_bytes, dk)) != BSATTN_OK) return rc;
+  if ((rc = check_strides(dv_strides, out_bytes, dv)) != BSATTN_OK) return rc;
   if (workspace == nullptr || workspace_bytes < bwd_workspace_bytes(B, H, N, D)) return BSATTN_ERR_WORKSPACE;
   AttnShape s;
   s.B = B; s.H = H; s.N = N; s.D = D; s.Bm = Bm; s.Hm = Hm; s.dtype = dtype; s.out_dtype = out_dtype;
   s.sm_scale = sm_scale;
-  for (int i = 0; i < 3; ++i) { s.qs[i] = q_strides[i]; s.ks[i] = k_strides[i]; s.vs[i] = v_strides[i]; s.os[i] = o_strides[i]; s.dos[i] = do_strides[i]; }
+  for (int i = 0; i < 3; ++i) { s.qs[i] = q_strides[i]; s.ks[i] = k_strides[i]; s.vs[i] = v_strides[i]; s.os[i] = o_strides[i]; s.dos[i] = do_strides[i];
+                               s.dqs[i] = dq_strides[i]; s.dks[i] = dk_strides[i]; s.dvs[i] = dv_strides[i]; }
   return launch_bwd(q, k, v, o, d_o, lse, dq, dk, dv, row_ptr, col_idx, col_ptr, row_idx, bits_rows, bits_cols, s,
                     workspace, (hipStream_t)stream);
 }
@@ -249,11 +260,12 @@ int bsattn_bwd(const void* q, const void* k, const void* v, const void* o, const
                const int32_t* col_idx, const int32_t* col_ptr, const int32_t* row_idx, int Bm, int Hm,
                int B, int H, int N, int D, int dtype, int out_dtype, float sm_scale,
                const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
-               const int64_t* o_strides, const int64_t* do_strides, void* workspace,
+               const int64_t* o_strides, const int64_t* do_strides, const int64_t* dq_strides,
+               const int64_t* dk_strides, const int64_t* dv_strides, void* workspace,
                size_t workspace_bytes, void* stream) {
   return bwd_common(q, k, v, o, d_o, lse, dq, dk, dv, row_ptr, col_idx, col_ptr, row_idx, nullptr, nullptr, Bm, Hm,
                     B, H, N, D, dtype, out_dtype, sm_scale, q_strides, k_strides, v_strides, o_strides, do_strides,
-                    workspace, workspace_bytes, stream);
+                    dq_strides, dk_strides, dv_strides, workspace, workspace_bytes, stream);
 }
 
 int bsattn_bwd_elementwise(const void* q, const void* k, const void* v, const void* o, const void* d_o,
@@ -262,13 +274,14 @@ int bsattn_bwd_elementwise(const void* q, const void* k, const void* v, const vo
                            const uint64_t* tile_bits_rows, const uint64_t* tile_bits_cols, int Bm, int Hm,
                            int B, int H, int N, int D, int dtype, int out_dtype, float sm_scale,
                            const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
-                           const int64_t* o_strides, const int64_t* do_strides, void* workspace,
+                           const int64_t* o_strides, const int64_t* do_strides, const int64_t* dq_strides,
+                           const int64_t* dk_strides, const int64_t* dv_strides, void* workspace,
                            size_t workspace_bytes, void* stream) {
   if (tile_bits_rows == nullptr || tile_bits_cols == nullptr) return BSATTN_ERR_NULL;
   if ((((uintptr_t)tile_bits_rows | (uintptr_t)tile_bits_cols) & 7) != 0) return BSATTN_ERR_STRIDE;
   return bwd_common(q, k, v, o, d_o, lse, dq, dk, dv, row_ptr, col_idx, col_ptr, row_idx, tile_bits_rows,
                     tile_bits_cols, Bm, Hm, B, H, N, D, dtype, out_dtype, sm_scale, q_strides, k_strides, v_strides,
-                    o_strides, do_strides, workspace, workspace_bytes, stream);
+                    o_strides, do_strides, dq_strides, dk_strides, dv_strides, workspace, workspace_bytes, stream);
 }
 
 int bsattn_reorder(const void* x, void* out, int BS, int NH, int F, int Hh, int W, int D, int elem_bytes,

@@ -34,6 +34,7 @@ struct BwdParams {
   float* part_dq; float* part_dk; float* part_dv;   // split > 1: fp32 partial results [split][B*H][N][D]
   float sm_scale, qk_scale;   // qk_scale = sm_scale * log2(e)
   int64_t qs[3], ks[3], vs[3], os[3], dos[3];
+  int64_t dqs[3], dks[3], dvs[3];   // batch, head, row strides of the results (elements)
 };
 
 constexpr float kLog2e = 1.4426950408889634f;
@@ -315,12 +316,13 @@ __global__ __launch_bounds__(128, D == 256 ? 1 : 2) void dq_kernel(const BwdPara
                          dqacc[db][4 * i4 + 2], dqacc[db][4 * i4 + 3]);
     return;
   }
-  void* base = prm.out_f32 ? (void*)((float*)prm.dq + (int64_t)bh * prm.N * D) : (void*)((unsigned short*)prm.dq + (int64_t)bh * prm.N * D);
+  const int64_t hoff = b * prm.dqs[0] + h * prm.dqs[1];
+  void* base = prm.out_f32 ? (void*)((float*)prm.dq + hoff) : (void*)((unsigned short*)prm.dq + hoff);
 #pragma unroll
   for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int i4 = 0; i4 < 4; ++i4)
-      store_out4<BF16>(base, qrow * D + 32 * db + 8 * i4 + 4 * g, prm.out_f32, dqacc[db][4 * i4] * prm.sm_scale,
+      store_out4<BF16>(base, qrow * prm.dqs[2] + 32 * db + 8 * i4 + 4 * g, prm.out_f32, dqacc[db][4 * i4] * prm.sm_scale,
                        dqacc[db][4 * i4 + 1] * prm.sm_scale, dqacc[db][4 * i4 + 2] * prm.sm_scale,
                        dqacc[db][4 * i4 + 3] * prm.sm_scale);
 }
@@ -587,17 +589,18 @@ __global__ __launch_bounds__(128, (QB == 1 && D == 64) ? 2 : 1) void dkdv_kernel
       }
     return;
   }
-  const int64_t hoff = (int64_t)bh * prm.N * D;
-  void* kbase = prm.out_f32 ? (void*)((float*)prm.dk + hoff) : (void*)((unsigned short*)prm.dk + hoff);
-  void* vbase = prm.out_f32 ? (void*)((float*)prm.dv + hoff) : (void*)((unsigned short*)prm.dv + hoff);
+  const int64_t koffh = b * prm.dks[0] + h * prm.dks[1], voffh = b * prm.dvs[0] + h * prm.dvs[1];
+  void* kbase = prm.out_f32 ? (void*)((float*)prm.dk + koffh) : (void*)((unsigned short*)prm.dk + koffh);
+  void* vbase = prm.out_f32 ? (void*)((float*)prm.dv + voffh) : (void*)((unsigned short*)prm.dv + voffh);
 #pragma unroll
   for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int i4 = 0; i4 < 4; ++i4) {
-      const int64_t off = krow * D + 32 * (DB0 + db) + 8 * i4 + 4 * g;
+      const int col = 32 * (DB0 + db) + 8 * i4 + 4 * g;
+      const int64_t off = krow * prm.dks[2] + col;
       store_out4<BF16>(kbase, off, prm.out_f32, dkacc[db][4 * i4] * prm.sm_scale, dkacc[db][4 * i4 + 1] * prm.sm_scale,
                        dkacc[db][4 * i4 + 2] * prm.sm_scale, dkacc[db][4 * i4 + 3] * prm.sm_scale);
-      store_out4<BF16>(vbase, off, prm.out_f32, dvacc[db][4 * i4], dvacc[db][4 * i4 + 1], dvacc[db][4 * i4 + 2],
+      store_out4<BF16>(vbase, krow * prm.dvs[2] + col, prm.out_f32, dvacc[db][4 * i4], dvacc[db][4 * i4 + 1], dvacc[db][4 * i4 + 2],
                        dvacc[db][4 * i4 + 3]);
     }
 }
@@ -606,15 +609,23 @@ __global__ __launch_bounds__(128, (QB == 1 && D == 64) ? 2 : 1) void dkdv_kernel
 // split > 1: out = scale * sum of the fp32 parts, rounded to the result type.  blockIdx.y: 0 dQ, 1 dK, 2 dV.
 // ---------------------------------------------------------------------------------------
 template <bool BF16>
-__global__ __launch_bounds__(256) void sum_parts_kernel(const BwdParams prm, int64_t quads) {
+__global__ __launch_bounds__(256) void sum_parts_kernel(const BwdParams prm, int64_t quads, int D) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;     // one thread per 4 consecutive values
   if (i >= quads) return;
   const float* part = blockIdx.y == 0 ? prm.part_dq : (blockIdx.y == 1 ? prm.part_dk : prm.part_dv);
   void* out = blockIdx.y == 0 ? prm.dq : (blockIdx.y == 1 ? prm.dk : prm.dv);
+  const int64_t* st = blockIdx.y == 0 ? prm.dqs : (blockIdx.y == 1 ? prm.dks : prm.dvs);
   const float scale = blockIdx.y == 2 ? 1.0f : prm.sm_scale;
   floatx4 acc = {0.f, 0.f, 0.f, 0.f};
   for (int c = 0; c < prm.split; ++c) acc += reinterpret_cast<const floatx4*>(part)[c * quads + i];
-  store_out4<BF16>(out, 4 * i, prm.out_f32, acc[0] * scale, acc[1] * scale, acc[2] * scale, acc[3] * scale);
+  // the parts are [B*H][N][D] without gaps; the result has its own strides
+  const int qpr = D / 4;                                   // quads per row
+  const int64_t row_all = i / qpr;
+  const int col = (int)(i - row_all * qpr) * 4;
+  const int bh = (int)(row_all / prm.N), row = (int)(row_all - (int64_t)bh * prm.N);
+  const int b = bh / prm.H, h = bh - b * prm.H;
+  store_out4<BF16>(out, b * st[0] + h * st[1] + row * st[2] + col, prm.out_f32, acc[0] * scale, acc[1] * scale,
+                   acc[2] * scale, acc[3] * scale);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -674,7 +685,7 @@ static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
   }
   if (prm.split > 1) {
     const int64_t quads = (int64_t)BH * prm.N * D / 4;
-    hipLaunchKernelGGL((sum_parts_kernel<BF16>), dim3((unsigned)((quads + 255) / 256), 3), dim3(256), 0, st, prm, quads);
+    hipLaunchKernelGGL((sum_parts_kernel<BF16>), dim3((unsigned)((quads + 255) / 256), 3), dim3(256), 0, st, prm, quads, D);
   }
 }
 
@@ -701,6 +712,7 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* o, const
   prm.qk_scale = s.sm_scale * kLog2e;
   for (int i = 0; i < 3; ++i) {
     prm.qs[i] = s.qs[i]; prm.ks[i] = s.ks[i]; prm.vs[i] = s.vs[i]; prm.os[i] = s.os[i]; prm.dos[i] = s.dos[i];
+    prm.dqs[i] = s.dqs[i]; prm.dks[i] = s.dks[i]; prm.dvs[i] = s.dvs[i];
   }
   const bool bf = s.dtype == BSATTN_BF16;
   // bf16 gradients are rounded to 8 bits anyway: P and dS are then rounded to bf16 as well (what the

@@ -29,6 +29,7 @@ struct AttnShape {
   int dtype, out_dtype;
   float sm_scale;
   int64_t qs[3], ks[3], vs[3], os[3], dos[3];  // batch, head, row strides (elements)
+  int64_t dqs[3], dks[3], dvs[3];              // ... of the backward's results
 };
 
 // attn_fwd.hip

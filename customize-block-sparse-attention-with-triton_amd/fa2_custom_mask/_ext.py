@@ -38,8 +38,8 @@ _SIGNATURES = {
     "bsattn_fwd_elementwise": ([_p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f,
                                 _p, _p, _p, _p, _p, ctypes.c_size_t, _p], _i),
     "bsattn_bwd_workspace": ([_i, _i, _i, _i, ctypes.POINTER(ctypes.c_size_t)], _i),
-    "bsattn_bwd": ([_p] * 13 + [_i] * 8 + [_f] + [_p] * 5 + [_p, ctypes.c_size_t, _p], _i),
-    "bsattn_bwd_elementwise": ([_p] * 15 + [_i] * 8 + [_f] + [_p] * 5 + [_p, ctypes.c_size_t, _p], _i),
+    "bsattn_bwd": ([_p] * 13 + [_i] * 8 + [_f] + [_p] * 8 + [_p, ctypes.c_size_t, _p], _i),
+    "bsattn_bwd_elementwise": ([_p] * 15 + [_i] * 8 + [_f] + [_p] * 8 + [_p, ctypes.c_size_t, _p], _i),
     "bsattn_reorder": ([_p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p], _i),
     "bsattn_mfma_rate_probe": ([_p, _i, _p, _p, _p], _i),
 }
@@ -95,15 +95,30 @@ def mask_lists_workspace(Bm, Hm, nb):
     return n.value
 
 
-@functools.lru_cache(maxsize=256)
-def fwd_workspace(B, H, N, D):
-    n = ctypes.c_size_t()
-    check(lib().bsattn_fwd_workspace(B, H, N, D, ctypes.byref(n)), "bsattn_fwd_workspace")
-    return n.value
+def _device_index(device):
+    """Index of `device` (a torch device or None = the current one); -1 without a GPU."""
+    if device is not None and getattr(device, "index", None) is not None:
+        return device.index
+    return torch.cuda.current_device() if torch.cuda.is_available() else -1
 
 
 @functools.lru_cache(maxsize=256)
-def bwd_workspace(B, H, N, D):
+def _workspace_on(which, B, H, N, D, index):
+    # the sizes depend on the device the library sees as current (its number of compute units)
     n = ctypes.c_size_t()
-    check(lib().bsattn_bwd_workspace(B, H, N, D, ctypes.byref(n)), "bsattn_bwd_workspace")
+    fn = getattr(lib(), which)
+    if index >= 0 and index != torch.cuda.current_device():
+        with torch.cuda.device(index):
+            rc = fn(B, H, N, D, ctypes.byref(n))
+    else:
+        rc = fn(B, H, N, D, ctypes.byref(n))
+    check(rc, which)
     return n.value
+
+
+def fwd_workspace(B, H, N, D, device=None):
+    return _workspace_on("bsattn_fwd_workspace", B, H, N, D, _device_index(device))
+
+
+def bwd_workspace(B, H, N, D, device=None):
+    return _workspace_on("bsattn_bwd_workspace", B, H, N, D, _device_index(device))

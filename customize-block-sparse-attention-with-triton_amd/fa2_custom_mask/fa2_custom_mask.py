@@ -34,6 +34,16 @@ def _prep(x):
     return x
 
 
+def _like(x, dtype):
+    """A result tensor laid out as the reference's torch.empty_like(x) lays it out (fa2_custom_mask.py:59,
+    101-103): the dimension order of x by stride, without gaps.  For q, k, v sliced out of one packed
+    [B, N, 3, H, D] tensor that is [B, N, H, D] order behind a [B, H, N, D] shape."""
+    t = torch.empty_like(x, dtype=dtype)
+    if t.stride(3) != 1 or any((s * t.element_size()) % 16 for s in t.stride()[:3]):
+        t = torch.empty(x.shape, dtype=dtype, device=x.device)
+    return t
+
+
 def _check_qkv(q, k, v, mask):
     if not (q.is_cuda and k.is_cuda and v.is_cuda):
         raise RuntimeError("q, k, v must be GPU tensors (there is no CPU path)")
@@ -75,7 +85,8 @@ def _dense_mask(device, nb):
     it: `groups` is unbound at fa2_custom_mask.py:69): one all-true block mask shared by all heads."""
     key = (device, nb)
     if key not in _all_true:
-        _all_true[key] = torch.ones((1, 1, nb, nb), dtype=torch.bool, device=device)
+        with torch.inference_mode(False):    # an ordinary tensor also when first asked for in inference mode: its lists are cached
+            _all_true[key] = torch.ones((1, 1, nb, nb), dtype=torch.bool, device=device)
     return _all_true[key]
 
 
@@ -121,9 +132,9 @@ def _use_quads(lists, B, H, N, D, wait=False):
 def _forward(q, k, v, lists, sm_scale, out_dtype, want_lse):
     B, H, N, D = q.shape
     q, k, v = _prep(q), _prep(k), _prep(v)
-    o = torch.empty((B, H, N, D), dtype=out_dtype, device=q.device)            # :59
+    o = _like(q, out_dtype)                                                     # :59
     lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device) if want_lse else None  # :70
-    wsb = _ext.fwd_workspace(B, H, N, D)
+    wsb = _ext.fwd_workspace(B, H, N, D, q.device)
     ws = torch.empty(wsb, dtype=torch.uint8, device=q.device)
     common = (lists.Bm, lists.Hm, B, H, N, D, _ext.dtype_code(q.dtype), _ext.dtype_code(out_dtype), float(sm_scale),
               _ext.strides4(q), _ext.strides4(k), _ext.strides4(v), _ext.strides4(o),
@@ -154,9 +165,9 @@ class ForwardPlan:
             raise ValueError("a plan takes whole tiles only: N % 64 == 0 and D in {64, 128, 256}")
         self.q, self.k, self.v, self.lists = _prep(q), _prep(k), _prep(v), lists
         out_dtype = out_dtype or q.dtype
-        self.o = torch.empty((B, H, N, D), dtype=out_dtype, device=q.device)
+        self.o = _like(self.q, out_dtype)
         self.lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device)
-        wsb = _ext.fwd_workspace(B, H, N, D)
+        wsb = _ext.fwd_workspace(B, H, N, D, q.device)
         self.ws = torch.empty(wsb, dtype=torch.uint8, device=q.device)
         self._keep = (_ext.strides4(self.q), _ext.strides4(self.k), _ext.strides4(self.v), _ext.strides4(self.o))
         stream = stream if stream is not None else torch.cuda.current_stream(q.device)
@@ -186,10 +197,8 @@ class ForwardPlan:
 def _backward(q, k, v, o, do, lse, lists, lists_t, sm_scale, out_dtype):
     B, H, N, D = q.shape
     q, k, v, o, do = _prep(q), _prep(k), _prep(v), _prep(o), _prep(do)
-    dq = torch.empty((B, H, N, D), dtype=out_dtype, device=q.device)           # :101-103
-    dk = torch.empty_like(dq)
-    dv = torch.empty_like(dq)
-    wsb = _ext.bwd_workspace(B, H, N, D)
+    dq, dk, dv = _like(q, out_dtype), _like(k, out_dtype), _like(v, out_dtype)   # :101-103
+    wsb = _ext.bwd_workspace(B, H, N, D, q.device)
     ws = torch.empty(wsb, dtype=torch.uint8, device=q.device)
     tensors = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(), lse.data_ptr(),
                dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
@@ -198,6 +207,7 @@ def _backward(q, k, v, o, do, lse, lists, lists_t, sm_scale, out_dtype):
     common = (lists.Bm, lists.Hm, B, H, N, D,
               _ext.dtype_code(q.dtype), _ext.dtype_code(out_dtype), float(sm_scale),
               _ext.strides4(q), _ext.strides4(k), _ext.strides4(v), _ext.strides4(o), _ext.strides4(do),
+              _ext.strides4(dq), _ext.strides4(dk), _ext.strides4(dv),
               ws.data_ptr(), wsb, _ext.current_stream(q.device))
     if lists.bits is None:
         rc = _ext.lib().bsattn_bwd(*tensors, *common)
@@ -219,12 +229,10 @@ class BackwardPlan:
         self.q, self.k, self.v, self.o, self.do = _prep(q), _prep(k), _prep(v), _prep(o), _prep(do)
         self.lse, self.lists, self.lists_t = lse, lists, lists_t
         out_dtype = out_dtype or q.dtype
-        self.dq = torch.empty((B, H, N, D), dtype=out_dtype, device=q.device)
-        self.dk = torch.empty_like(self.dq)
-        self.dv = torch.empty_like(self.dq)
-        wsb = _ext.bwd_workspace(B, H, N, D)
+        self.dq, self.dk, self.dv = _like(self.q, out_dtype), _like(self.k, out_dtype), _like(self.v, out_dtype)
+        wsb = _ext.bwd_workspace(B, H, N, D, q.device)
         self.ws = torch.empty(wsb, dtype=torch.uint8, device=q.device)
-        self._keep = tuple(_ext.strides4(t) for t in (self.q, self.k, self.v, self.o, self.do))
+        self._keep = tuple(_ext.strides4(t) for t in (self.q, self.k, self.v, self.o, self.do, self.dq, self.dk, self.dv))
         stream = stream if stream is not None else torch.cuda.current_stream(q.device)
         self._args = (self.q.data_ptr(), self.k.data_ptr(), self.v.data_ptr(), self.o.data_ptr(), self.do.data_ptr(),
                       lse.data_ptr(), self.dq.data_ptr(), self.dk.data_ptr(), self.dv.data_ptr(),

@@ -212,18 +212,41 @@ class _ListsCache:
 
     def __init__(self, capacity=8):
         self.capacity = capacity
-        self._entries = []     # (weakref to mask, version, N, transpose, lists), most recent last
+        # (weakref to mask, version, N, transpose, lists, stream the lists were built on, event), most recent last
+        self._entries = []
+
+    @staticmethod
+    def _version(mask):
+        """The tensor's write counter, or None for a tensor that keeps none (one created under
+        torch.inference_mode()): writes to such a tensor cannot be seen, so it is never cached."""
+        try:
+            return mask._version
+        except RuntimeError:
+            return None
 
     def get(self, mask, N, transpose):
-        for i, (ref, ver, n, tr, lists) in enumerate(self._entries):
-            if ref() is mask and ver == mask._version and n == N and tr == transpose:
+        version = self._version(mask)
+        if version is None:
+            return None
+        for i, (ref, ver, n, tr, lists, stream, ready) in enumerate(self._entries):
+            if ref() is mask and ver == version and n == N and tr == transpose:
                 self._entries.append(self._entries.pop(i))
+                # the lists were filled by kernels on `stream`: work on another stream waits for them
+                current = torch.cuda.current_stream(mask.device)
+                if current != stream:
+                    current.wait_event(ready)
                 return lists
         return None
 
     def put(self, mask, N, transpose, lists):
+        version = self._version(mask)
+        if version is None:
+            return
+        stream = torch.cuda.current_stream(mask.device)
+        ready = torch.cuda.Event()
+        ready.record(stream)
         self._entries = [e for e in self._entries if e[0]() is not None]
-        self._entries.append((weakref.ref(mask), mask._version, N, transpose, lists))
+        self._entries.append((weakref.ref(mask), version, N, transpose, lists, stream, ready))
         del self._entries[:-self.capacity]
 
     def clear(self):

@@ -233,7 +233,9 @@ int bsattn_fwd_elementwise(const void* q, const void* k, const void* v, void* o,
 int bsattn_bwd_workspace(int B, int H, int N, int D, size_t* bytes);
 
 /* q,k,v,o,d_o: [B,H,N,D] fp16/bf16 with their own strides; lse from bsattn_fwd.
- * dq,dk,dv: [B,H,N,D] of out_dtype, contiguous.
+ * dq,dk,dv: [B,H,N,D] of out_dtype with strides dq_strides, dk_strides, dv_strides (innermost 1;
+ *        NULL: no gaps), e.g. the three slices of one packed [B,N,3,H,D] gradient buffer, as the
+ *        reference's torch.empty_like(q) gives for such inputs (fa2_custom_mask.py:101-103).
  * row_ptr/col_idx: row lists; col_ptr/row_idx: column lists (the same call with the mask's
  * row and column strides swapped). */
 int bsattn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
@@ -243,6 +245,7 @@ int bsattn_bwd(const void* q, const void* k, const void* v, const void* o, const
                int B, int H, int N, int D, int dtype, int out_dtype, float sm_scale,
                const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
                const int64_t* o_strides, const int64_t* do_strides,
+               const int64_t* dq_strides, const int64_t* dk_strides, const int64_t* dv_strides,
                void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------
@@ -259,8 +262,9 @@ int bsattn_bwd_elementwise(const void* q, const void* k, const void* v, const vo
                            int Bm, int Hm, int B, int H, int N, int D, int dtype, int out_dtype,
                            float sm_scale, const int64_t* q_strides, const int64_t* k_strides,
                            const int64_t* v_strides, const int64_t* o_strides,
-                           const int64_t* do_strides, void* workspace, size_t workspace_bytes,
-                           void* stream);
+                           const int64_t* do_strides, const int64_t* dq_strides,
+                           const int64_t* dk_strides, const int64_t* dv_strides, void* workspace,
+                           size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------
  * Head-wise token reorder.  Replaces reorder_kernel / inv_reorder_kernel

@@ -6,8 +6,9 @@
  *   oracle_naive_fwd      kernel-test.py:37-40 with the mask expansion of :18
  *   oracle_reorder        fa2_custom_mask/permute.py:5-58
  *   oracle_inv_reorder    fa2_custom_mask/permute.py:60-126
- * Pinned by tests/test_oracle_c.py against the numpy oracle, which is itself pinned
- * against library closed forms and the hand-worked fixture.
+ * Pinned against the numpy oracle, which is itself pinned against library closed forms and
+ * the hand-worked fixture: tests/test_oracle_index.py (oracle_build_groups),
+ * tests/test_oracle_attention.py (oracle_naive_fwd), tests/test_oracle_reorder.py (the reorders).
  */
 #include <math.h>
 #include <stdint.h>

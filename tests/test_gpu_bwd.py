@@ -132,3 +132,76 @@ def test_backward_plan_matches_the_call(dev):
     with pytest.raises(ValueError):
         fm.BackwardPlan(q[:, :, :100], k[:, :, :100], v[:, :, :100], o[:, :, :100], do[:, :, :100], lse[:, :, :100],
                         lists, lists_t, sc)
+
+
+@pytest.mark.parametrize("out_fp32", [False, True])
+def test_packed_qkv_layout_is_kept(dev, out_fp32):
+    """q, k, v sliced out of one packed [B, N, 3, H, D] tensor (no copies): o, dq, dk, dv come back in the
+    layout torch.empty_like gives for such inputs, which is what the reference allocates
+    (fa2_custom_mask.py:59, 101-103), and the kernels write through those strides."""
+    import fa2_custom_mask as fm
+    B, H, N, D = 2, 3, 512, 64
+    g = torch.Generator().manual_seed(41)
+    qkv = torch.randn(B, N, 3, H, D, generator=g).to(torch.float16)
+    do = torch.randn(B, N, H, D, generator=g).to(torch.float16)
+    mask = uniform_block_mask(1, 3, 8, 0.4, 9)
+    sc = 0.125
+    qkv_d, do_d = qkv.to(dev), do.to(dev)
+    q, k, v = [qkv_d[:, :, i].transpose(1, 2) for i in range(3)]          # [B, H, N, D] views
+    assert not q.is_contiguous()
+    o, lse, dq, dk, dv = fm.attention_forward_backward(q, k, v, mask.to(dev), sc, do_d.transpose(1, 2), out_fp32=out_fp32)
+    torch.cuda.synchronize()
+    want = torch.empty_like(q, dtype=torch.float32 if out_fp32 else torch.float16).stride()
+    assert want == (N * H * D, D, H * D, 1)
+    for t in (o, dq, dk, dv):
+        assert t.stride() == want
+    qc, kc, vc = [f32(qkv[:, :, i].transpose(1, 2).contiguous()) for i in range(3)]
+    doc = f32(do.transpose(1, 2).contiguous())
+    dq_r, dk_r, dv_r, _ = orc.attention_backward(qc, kc, vc, mask.numpy(), sc, doc)
+    o_r = orc.naive_attention(qc, kc, vc, mask.numpy(), sc)
+    for got, ref in ((o, o_r), (dq, dq_r), (dk, dk_r), (dv, dv_r)):
+        ma, rl = errors(got, ref)
+        assert ma <= 2e-2 and rl <= 1e-3
+
+
+def test_packed_qkv_split_lists(dev):
+    """The same for a single long head, whose row and column lists are walked by several workgroups (the
+    gradients are then summed from fp32 parts by a kernel of its own, which writes through the strides)."""
+    import fa2_custom_mask as fm
+    B, H, N, D = 1, 1, 2048, 64
+    g = torch.Generator().manual_seed(42)
+    qkv = torch.randn(B, N, 3, H, D, generator=g).to(torch.float16)
+    do = torch.randn(B, H, N, D, generator=g).to(torch.float16)
+    mask = uniform_block_mask(1, 1, 32, 0.5, 10)
+    qkv_d = qkv.to(dev)
+    q, k, v = [qkv_d[:, :, i].transpose(1, 2) for i in range(3)]
+    o, lse, dq, dk, dv = fm.attention_forward_backward(q, k, v, mask.to(dev), 0.125, do.to(dev))
+    torch.cuda.synchronize()
+    qc, kc, vc = [f32(qkv[:, :, i].transpose(1, 2).contiguous()) for i in range(3)]
+    dq_r, dk_r, dv_r, _ = orc.attention_backward(qc, kc, vc, mask.numpy(), 0.125, f32(do))
+    for got, ref in ((dq, dq_r), (dk, dk_r), (dv, dv_r)):
+        assert got.stride() == torch.empty_like(q).stride()
+        ma, rl = errors(got, ref)
+        assert ma <= 2e-2 and rl <= 1e-3
+
+
+def test_delta_against_oracle(dev):
+    """delta = rowsum(O * dO) (fa2_bwd.py:17), the first step of the backward, lives at the start of the
+    workspace: compared with the oracle's directly, not only through the gradients."""
+    import fa2_custom_mask as fm
+    B, H, N, D = 2, 2, 1024, 128
+    q, k, v, do = make_qkv(B, H, N, D, torch.float16, 43, n=4)
+    mask = uniform_block_mask(1, 1, 16, 0.4, 11)
+    sc = 1.0 / np.sqrt(D)
+    lists = fm.block_mask_to_lists(mask.to(dev))
+    lists_t = fm.block_mask_to_lists(mask.to(dev), transpose=True)
+    qd, kd, vd, dod = [x.to(dev) for x in (q, k, v, do)]
+    o, lse = fm.ForwardPlan(qd, kd, vd, lists, sc).run()
+    plan = fm.BackwardPlan(qd, kd, vd, o, dod, lse, lists, lists_t, sc)
+    plan.run()
+    torch.cuda.synchronize()
+    delta = plan.ws[:B * H * N * 4].view(torch.float32).reshape(B, H, N).cpu().numpy()
+    _, _, _, delta_r = orc.attention_backward(f32(q), f32(k), f32(v), mask.numpy(), sc, f32(do))
+    # O enters as the fp16-rounded forward result: 2^-11 relative per term, D terms of random sign
+    assert np.abs(delta - delta_r).max() <= 5e-3
+    assert np.linalg.norm(delta - delta_r) / np.linalg.norm(delta_r) <= 2e-3

@@ -250,3 +250,55 @@ def test_invariants_large(dev):
     mean_rows = (w @ vt) / w.sum(1, keepdim=True)
     ref = mean_rows.repeat_interleave(64, 0)
     assert float((o[0, 0].float() - ref).abs().max()) <= 2e-3
+
+
+def test_inference_mode(dev):
+    """Tensors made under torch.inference_mode() keep no write counter (reading it raises): the cache of
+    kept-tile lists must not depend on it.  Block mask, elementwise mask and no mask, each called
+    twice, with the mask changed in place between the two calls."""
+    import fa2_custom_mask as fm
+    B, H, N, D = 1, 2, 512, 64
+    q, k, v = make_qkv(B, H, N, D, torch.float16, 31)
+    sm_scale = 0.125
+    with torch.inference_mode():
+        qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+        block = uniform_block_mask(1, 2, 8, 0.5, 6).to(dev)
+        g = torch.Generator().manual_seed(7)
+        dense = (torch.rand(1, 1, N, N, generator=g) < 0.3) | torch.eye(N, dtype=torch.bool)
+        dense_d = dense.to(dev)
+        for _ in range(2):
+            o = fm.flash_attention_custom_mask(qd, kd, vd, block, sm_scale)
+            o_ref = orc.naive_attention(f32(q), f32(k), f32(v), block.cpu().numpy(), sm_scale)
+            assert errors(o, o_ref)[1] <= RELL2
+            block[0, 0, 2, :] = False            # a write the cache cannot see on such a tensor
+            block[0, 0, 2, 5] = True
+        for _ in range(2):
+            o = fm.flash_attention_custom_mask(qd, kd, vd, dense_d, sm_scale)
+            o_ref = orc.naive_attention(f32(q), f32(k), f32(v), dense_d.cpu().numpy(), sm_scale)
+            assert errors(o, o_ref)[1] <= RELL2
+            dense_d[0, 0, 100:200, 0:300] = False
+            dense_d[0, 0, 100:200, 7] = True
+        for _ in range(2):
+            o = fm.flash_attention_custom_mask(qd, kd, vd, None, sm_scale)
+            o_ref = orc.naive_attention(f32(q), f32(k), f32(v), np.ones((1, 1, 8, 8), dtype=bool), sm_scale)
+            assert errors(o, o_ref)[1] <= RELL2
+
+
+def test_cached_lists_on_another_stream(dev):
+    """The lists of a mask are built on the stream of the first call; a call on another stream uses the
+    cached lists only after that work (the cache makes the second stream wait)."""
+    import fa2_custom_mask as fm
+    B, H, N, D = 1, 1, 4096, 64
+    q, k, v = make_qkv(B, H, N, D, torch.float16, 32)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    mask = uniform_block_mask(1, 1, 64, 0.3, 8)
+    o_ref = orc.naive_attention(f32(q), f32(k), f32(v), mask.numpy(), 0.125)
+    md = mask.to(dev)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream(dev)
+    o1 = fm.flash_attention_custom_mask(qd, kd, vd, md, 0.125)          # builds the lists on the current stream
+    with torch.cuda.stream(side):
+        o2 = fm.flash_attention_custom_mask(qd, kd, vd, md, 0.125)      # cached lists, other stream
+    side.synchronize()
+    torch.cuda.synchronize()
+    assert errors(o1, o_ref)[1] <= RELL2 and errors(o2, o_ref)[1] <= RELL2
