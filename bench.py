@@ -13,7 +13,8 @@ import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-sys.path.insert(0, os.path.join(ROOT, "customize-block-sparse-attention-with-triton_amd"))
+PKG = os.path.join(ROOT, "customize-block-sparse-attention-with-triton_amd")
+sys.path.insert(0, PKG)
 sys.path.insert(0, ROOT)
 
 N, D, TILE = 17536, 64, 64
@@ -127,10 +128,15 @@ def reorder_case(torch, dev, fm):
 
 
 def mfma_ceiling(torch, dev, iters=8192, launches=10):
-    """Sustained fp16 MFMA rate (TFLOP/s) of bsattn_mfma_rate_probe for two operand patterns."""
+    """Sustained fp16 MFMA rate (TFLOP/s) for two operand patterns, measured with the probe library
+    (probe/mfma_rate.hip in the package directory, built by build.py beside the attention library)."""
     import ctypes
-    from fa2_custom_mask import _ext
-    lib = _ext.lib()
+    path = os.path.join(PKG, "probe", "libbsattn_probe.so")
+    if not os.path.exists(path):
+        raise RuntimeError("libbsattn_probe.so not found at %s: run build.py" % path)
+    lib = ctypes.CDLL(path)
+    lib.probe_mfma_rate.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    lib.probe_mfma_rate.restype = ctypes.c_int
     sink = torch.empty(512, dtype=torch.float32, device=dev)
     st = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
     g = torch.Generator().manual_seed(7)
@@ -141,8 +147,9 @@ def mfma_ceiling(torch, dev, iters=8192, launches=10):
         flops = ctypes.c_double()
 
         def run():
-            _ext.check(lib.bsattn_mfma_rate_probe(ops.data_ptr(), iters, sink.data_ptr(),
-                                                  ctypes.byref(flops), st), "bsattn_mfma_rate_probe")
+            rc = lib.probe_mfma_rate(ops.data_ptr(), iters, sink.data_ptr(), ctypes.byref(flops), st)
+            if rc != 0:
+                raise RuntimeError("probe_mfma_rate failed with %d" % rc)
         ts = event_times(run, launches, 3, torch)
         out[name + "_tflops"] = round(flops.value / (ts[len(ts) // 2] * 1e-3) / 1e12, 1)
     out["unit"] = "TFLOP/s"

@@ -294,11 +294,4 @@ int bsattn_reorder(const void* x, void* out, int BS, int NH, int F, int Hh, int 
   return launch_reorder(x, out, BS, NH, F, Hh, W, (int)row_bytes, orders, inv_orders, (hipStream_t)stream);
 }
 
-int bsattn_mfma_rate_probe(const void* operands, int iters, float* sink, double* flops, void* stream) {
-  if (operands == nullptr || sink == nullptr) return BSATTN_ERR_NULL;
-  if (iters <= 0 || iters > (1 << 20)) return BSATTN_ERR_RANGE;
-  if (((uintptr_t)operands & 15) != 0) return BSATTN_ERR_STRIDE;
-  return launch_mfma_rate(operands, iters, sink, flops, (hipStream_t)stream);
-}
-
 }  // extern "C"

@@ -77,9 +77,6 @@ int launch_bwd(const void* q, const void* k, const void* v, const void* o, const
 int launch_reorder(const void* x, void* out, int BS, int NH, int F, int Hh, int W, int row_bytes,
                    const int32_t* orders, const int32_t* inv_orders, hipStream_t st);
 
-// calibrate.hip
-int launch_mfma_rate(const void* operands, int iters, float* sink, double* flops, hipStream_t st);
-
 inline int launch_status() { return hipGetLastError() == hipSuccess ? BSATTN_OK : BSATTN_ERR_LAUNCH; }
 
 }  // namespace bsattn

@@ -41,7 +41,6 @@ _SIGNATURES = {
     "bsattn_bwd": ([_p] * 13 + [_i] * 8 + [_f] + [_p] * 8 + [_p, ctypes.c_size_t, _p], _i),
     "bsattn_bwd_elementwise": ([_p] * 15 + [_i] * 8 + [_f] + [_p] * 8 + [_p, ctypes.c_size_t, _p], _i),
     "bsattn_reorder": ([_p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p], _i),
-    "bsattn_mfma_rate_probe": ([_p, _i, _p, _p, _p], _i),
 }
 EXPORTS = tuple(_SIGNATURES)
 

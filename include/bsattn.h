@@ -278,19 +278,6 @@ int bsattn_reorder(const void* x, void* out, int BS, int NH, int F, int Hh, int 
                    int elem_bytes, const int32_t* orders, const int32_t* inv_orders,
                    void* stream);
 
-/* ------------------------------------------------------------------------------------
- * Measurement aid with no counterpart in the reference: the matrix-core rate the GPU
- * sustains for given operand data.  One workgroup of 8 wavefronts per compute unit; every
- * wavefront issues iters x 8 MFMAs (32x32x16 fp16, fp32 accumulate) whose operand
- * fragments are read from `operands` (8192 bytes of device memory, 16-byte aligned:
- * 64 lanes x 8 fragments x 8 fp16).  sink: 512 floats of device memory (keeps the work
- * alive).  *flops (host memory, may be NULL) receives the floating-point operations of
- * the launch; time the launch with events on `stream` to obtain the rate.  The rate
- * depends on the operand data (bit toggling -> power -> clock), which is the point.
- * ---------------------------------------------------------------------------------- */
-int bsattn_mfma_rate_probe(const void* operands, int iters, float* sink, double* flops,
-                           void* stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -71,17 +71,6 @@ def test_argument_validation_without_gpu():
     assert l.bsattn_reorder(P, P, 1, 1, 2, 2, 2, 4, 2, None, None, None) == -1
 
 
-def test_mfma_rate_probe_validation_without_gpu():
-    from fa2_custom_mask import _ext
-    l = _ext.lib()
-    P = ctypes.c_void_p(4096)
-    assert l.bsattn_mfma_rate_probe(None, 16, P, None, None) == -1      # BSATTN_ERR_NULL
-    assert l.bsattn_mfma_rate_probe(P, 16, None, None, None) == -1
-    assert l.bsattn_mfma_rate_probe(P, 0, P, None, None) == -8          # BSATTN_ERR_RANGE
-    assert l.bsattn_mfma_rate_probe(P, 1 << 21, P, None, None) == -8
-    assert l.bsattn_mfma_rate_probe(ctypes.c_void_p(4100), 16, P, None, None) == -5   # BSATTN_ERR_STRIDE (alignment)
-
-
 def test_python_wrapper_rejects_bad_input_without_gpu():
     import torch
     import fa2_custom_mask as fm
@@ -94,17 +83,3 @@ def test_python_wrapper_rejects_bad_input_without_gpu():
     with pytest.raises(RuntimeError):
         fm.build_groups_from_block_mask(m)                                       # CPU mask: no CPU path
 
-
-def test_quad_split_arithmetic(tmp_path):
-    """The work split of the forward kernel that walks quads (csrc/fwd_quad_split.h) is plain integer
-    arithmetic shared with the kernel: a host program checks on random weight axes that the ranges
-    tile the axis and that every quad's parts are the ranges quad_parts() names (built with the
-    address and undefined-behaviour sanitizers)."""
-    import subprocess
-    exe = str(tmp_path / "quad_split_check")
-    src = os.path.join(ROOT, "tests", "quad_split_check.cpp")
-    inc = os.path.join(ROOT, "customize-block-sparse-attention-with-triton_amd", "csrc")
-    subprocess.run(["g++", "-O1", "-std=c++17", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
-                    "-static-libasan", "-I" + inc, src, "-o", exe], check=True)
-    out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout
-    assert out.startswith("ok ")

@@ -119,15 +119,21 @@ def test_c5_fwd_bwd_bf16_d128(dev):
 
 
 def test_mfma_rate_probe_runs(dev):
-    """The measurement aid launches, reports the FLOPs of the launch and leaves finite sums."""
+    """The benchmark's measurement aid (a library of its own, not part of the attention library) launches,
+    reports the FLOPs of the launch and leaves the expected sums."""
     import ctypes
+    import os
     from fa2_custom_mask import _ext
-    lib = _ext.lib()
+    path = os.path.join(os.path.dirname(os.path.dirname(_ext.LIB_PATH)), "probe", "libbsattn_probe.so")
+    lib = ctypes.CDLL(path)
+    lib.probe_mfma_rate.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     ops = torch.ones(4096, dtype=torch.float16, device=dev)
     sink = torch.full((512,), float("nan"), dtype=torch.float32, device=dev)
     flops = ctypes.c_double()
     st = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
-    rc = lib.bsattn_mfma_rate_probe(ops.data_ptr(), 4, sink.data_ptr(), ctypes.byref(flops), st)
+    assert lib.probe_mfma_rate(None, 16, sink.data_ptr(), None, st) == -1
+    assert lib.probe_mfma_rate(ops.data_ptr(), 0, sink.data_ptr(), None, st) == -8
+    rc = lib.probe_mfma_rate(ops.data_ptr(), 4, sink.data_ptr(), ctypes.byref(flops), st)
     assert rc == 0
     torch.cuda.synchronize()
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
