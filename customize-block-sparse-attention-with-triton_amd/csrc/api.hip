@@ -40,7 +40,7 @@ int bsattn_mask_lists_workspace(int Bm, int Hm, int nb, size_t* bytes) {
   if (bytes == nullptr) return BSATTN_ERR_NULL;
   if (Bm <= 0 || Hm <= 0 || nb <= 0) return BSATTN_ERR_SHAPE;
   if ((int64_t)Bm * Hm * nb * nb > 0x7fffffffLL) return BSATTN_ERR_RANGE;
-  *bytes = (size_t)Bm * Hm * nb * 2 * sizeof(int32_t);
+  *bytes = (size_t)Bm * Hm * nb * 2 * sizeof(int32_t);     // per row: count, position in `groups`
   return BSATTN_OK;
 }
 
@@ -53,6 +53,7 @@ int bsattn_block_mask_to_lists(const uint8_t* block, int Bm, int Hm, int nb, int
   const int rc = bsattn_mask_lists_workspace(Bm, Hm, nb, &need);
   if (rc != BSATTN_OK) return rc;
   if (workspace == nullptr || workspace_bytes < need) return BSATTN_ERR_WORKSPACE;
+  if (((uintptr_t)workspace & 3) != 0) return BSATTN_ERR_STRIDE;
   return launch_block_mask_to_lists(block, Bm, Hm, nb, sb, sh, sm, sn, row_ptr, col_idx, groups, counts,
                                     (int32_t*)workspace, (hipStream_t)stream);
 }

@@ -842,7 +842,7 @@ void fwd_kernel(const FwdParams prm) {
 
 // A 48-bit number that differs from launch to launch (and, through its start value, from process
 // to process); never zero.
-static unsigned long long next_epoch() {
+unsigned long long next_epoch() {
   static std::atomic<unsigned long long> counter{
       (unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count() * 0x9E3779B97F4A7C15ull};
   unsigned long long e;

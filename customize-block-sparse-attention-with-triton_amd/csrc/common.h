@@ -48,6 +48,7 @@ inline void once_per_device(std::atomic<unsigned long long>& done, F&& f) {
   done.fetch_or(bit, std::memory_order_release);
 }
 size_t fwd_workspace_bytes(int B, int H, int N, int D);
+unsigned long long next_epoch();   // a 48-bit number that differs from launch to launch, never zero
 int set_deterministic(int on);   // returns the previous setting
 int get_deterministic();
 int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,

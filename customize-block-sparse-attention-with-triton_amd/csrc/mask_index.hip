@@ -211,33 +211,93 @@ int launch_quad_lists(const int32_t* row_ptr, const int32_t* col_idx, int Bm, in
 // lists both transposed, the words describe the columns (what the dK/dV pass needs).
 // ---------------------------------------------------------------------------------------
 constexpr int PACK_SPLIT = 8;
+constexpr int PACK_G = 4;     // measured against 8 and 16: fewer, longer wavefronts lose more than longer runs gain
+
+// 16 bool bytes (each 0 or 1) -> 16 bits: a dot product of four bytes with (1, 2, 4, 8) or (16, 32, 64, 128)
+// places four bits at once
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ unsigned bools16(const u32x4& d) {
+  const unsigned lo = __builtin_amdgcn_udot4(d[1], 0x80402010u, __builtin_amdgcn_udot4(d[0], 0x08040201u, 0u, false), false);
+  const unsigned hi = __builtin_amdgcn_udot4(d[3], 0x80402010u, __builtin_amdgcn_udot4(d[2], 0x08040201u, 0u, false), false);
+  return lo | (hi << 8);
+}
+
+// MODE 0: columns are contiguous in memory (sn == 1); MODE 1: rows are (sm == 1: the call for the column
+// lists, with the mask's strides swapped); MODE 2: neither (one byte per load, one tile per wavefront).
+// MODE 0 / 1: a tile is 64 memory rows of 64 contiguous bytes, half a 128-byte line of the L2, whose other
+// half belongs to the neighbouring tile, and a small piece of a DRAM page.  A wavefront therefore takes G
+// consecutive entries of the list at a time (in a dense stretch of a row list: 64 G contiguous bytes per
+// memory row): one load instruction covers 16 / G memory rows of the G tiles, 16 bytes per lane.  The four
+// lanes that share a memory row of a tile put their bits together, the words go through LDS so that lane l
+// ends up with the word of memory row l of each tile.  In MODE 1 that is bit r of the words to come for
+// column l: the 64 x 64 bit matrix is transposed with one ballot per word.
+template <int MODE, int G>
 __global__ __launch_bounds__(256) void pack_tiles_kernel(const uint8_t* __restrict__ dense, int nb, int H,
                                                          int64_t sb, int64_t sh, int64_t sm, int64_t sn,
                                                          const int32_t* __restrict__ row_ptr,
                                                          const int32_t* __restrict__ col_idx,
                                                          uint8_t* __restrict__ partial,
                                                          unsigned long long* __restrict__ bits) {
+  __shared__ unsigned long long stage[MODE == 2 ? 1 : 4][MODE == 2 ? 1 : G][64];      // [wavefront][tile of the group][memory row]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int rb = blockIdx.x / PACK_SPLIT, sub = blockIdx.x % PACK_SPLIT, bh = blockIdx.y;
+  // (row blocks from the last to the first: with causal masks the long lists then start first)
+  const int rb = nb - 1 - blockIdx.x / PACK_SPLIT, sub = blockIdx.x % PACK_SPLIT, bh = blockIdx.y;
   const int32_t* rp = row_ptr + (int64_t)bh * nb;
   const int t0 = rp[rb], t1 = rp[rb + 1];
-  const uint8_t* rowp = dense + (bh / H) * sb + (bh % H) * sh + ((int64_t)rb * 64 + lane) * sm;
-  for (int t = t0 + sub * 4 + wave; t < t1; t += 4 * PACK_SPLIT) {
-    const uint8_t* p = rowp + (int64_t)col_idx[t] * 64 * sn;
-    unsigned long long word = 0ull;
-    if (sn == 1) {
-      // 4 bool bytes -> 4 bits with one multiplication (bytes are 0 or 1)
-#pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        const unsigned int d = *reinterpret_cast<const unsigned int*>(p + 4 * j);
-        word |= (unsigned long long)(((d * 0x01020408u) >> 24) & 0xFu) << (4 * j);
-      }
-    } else {
+  const uint8_t* head = dense + (bh / H) * sb + (bh % H) * sh + (int64_t)rb * 64 * sm;
+  if constexpr (MODE == 2) {
+    for (int t = t0 + sub * 4 + wave; t < t1; t += 4 * PACK_SPLIT) {
+      const uint8_t* p = head + (int64_t)col_idx[t] * 64 * sn + lane * sm;
+      unsigned long long word = 0ull;
       for (int c = 0; c < 64; ++c) word |= (unsigned long long)(p[(int64_t)c * sn] != 0) << c;
+      bits[(int64_t)t * 64 + lane] = word;
+      const bool full = __ballot(word == ~0ull) == ~0ull;
+      if (lane == 0) partial[t] = full ? 0 : 1;
     }
-    bits[(int64_t)t * 64 + lane] = word;
-    const bool full = __ballot(word == ~0ull) == ~0ull;
-    if (lane == 0) partial[t] = full ? 0 : 1;
+  } else {
+    constexpr int RPI = 16 / G;                      // memory rows per load instruction
+    const int64_t S = MODE == 0 ? sm : sn;           // stride between memory rows (the other stride is 1)
+    const int64_t step = 64 * sn;                    // offset of a tile = its column block times this
+    const int sub_row = lane / (4 * G), j = (lane >> 2) % G, chunk = lane & 3;
+    unsigned long long (*my)[64] = stage[wave];
+    for (int tg = t0 + G * (sub * 4 + wave); tg < t1; tg += 4 * G * PACK_SPLIT) {
+      const int tj = tg + j < t1 ? tg + j : t1 - 1;               // (a group past the end repeats the last tile)
+      const uint8_t* p = head + (int64_t)col_idx[tj] * step + (int64_t)sub_row * S + 16 * chunk;
+#pragma unroll 1
+      for (int r0 = 0; r0 < 64; r0 += 16 * RPI) {                 // 16 loads in flight
+        u32x4 d[16];
+#pragma unroll
+        for (int it = 0; it < 16; ++it)
+          d[it] = *reinterpret_cast<const u32x4*>(p + (r0 + RPI * it) * S);   // (cached: a neighbour wants the other half line)
+#pragma unroll
+        for (int it = 0; it < 16; ++it) {
+          // the 16 bits of the four lanes that share the memory row, side by side (lane 4k + c holds bits 16c ..)
+          const unsigned h = bools16(d[it]);
+          const unsigned h0 = __builtin_amdgcn_mov_dpp(h, 0x00, 0xf, 0xf, true), h1 = __builtin_amdgcn_mov_dpp(h, 0x55, 0xf, 0xf, true);
+          const unsigned h2 = __builtin_amdgcn_mov_dpp(h, 0xaa, 0xf, 0xf, true), h3 = __builtin_amdgcn_mov_dpp(h, 0xff, 0xf, 0xf, true);
+          const unsigned long long x = (unsigned long long)(h0 | (h1 << 16)) | ((unsigned long long)(h2 | (h3 << 16)) << 32);
+          if (chunk == 0) my[j][r0 + RPI * it + sub_row] = x;    // word of that memory row of tile j
+        }
+      }
+      // (the LDS operations of one wavefront complete in order: the reads below see the writes above)
+#pragma unroll 1
+      for (int jj = 0; jj < G; ++jj) {
+        if (tg + jj >= t1) break;
+        unsigned long long word = my[jj][lane];
+        if constexpr (MODE == 1) {
+          unsigned long long out = 0ull;
+#pragma unroll 8
+          for (int r = 0; r < 64; ++r) {
+            const unsigned long long b = __ballot((word >> r) & 1ull);
+            if (lane == r) out = b;
+          }
+          word = out;
+        }
+        bits[(int64_t)(tg + jj) * 64 + lane] = word;
+        const bool full = __ballot(word == ~0ull) == ~0ull;
+        if (lane == 0) partial[tg + jj] = full ? 0 : 1;
+      }
+    }
   }
 }
 
@@ -297,8 +357,15 @@ int launch_tail_tiles(int Bm, int Hm, int nb, int valid, int transpose, const in
 int launch_pack_tiles(const uint8_t* dense, int Bm, int Hm, int nb, int64_t sb, int64_t sh, int64_t sm,
                       int64_t sn, const int32_t* row_ptr, const int32_t* col_idx, uint8_t* partial,
                       unsigned long long* bits, hipStream_t st) {
-  hipLaunchKernelGGL(pack_tiles_kernel, dim3(nb * PACK_SPLIT, Bm * Hm), dim3(256), 0, st, dense, nb, Hm, sb, sh, sm, sn,
-                     row_ptr, col_idx, partial, bits);
+  // the wide loads need 16-byte aligned memory rows
+  const bool wide = (((uintptr_t)dense | (uintptr_t)sb | (uintptr_t)sh) & 15) == 0;
+  const dim3 grid(nb * PACK_SPLIT, Bm * Hm);
+  if (wide && sn == 1 && sm % 16 == 0)
+    hipLaunchKernelGGL((pack_tiles_kernel<0, PACK_G>), grid, dim3(256), 0, st, dense, nb, Hm, sb, sh, sm, sn, row_ptr, col_idx, partial, bits);
+  else if (wide && sm == 1 && sn % 16 == 0)
+    hipLaunchKernelGGL((pack_tiles_kernel<1, 4>), grid, dim3(256), 0, st, dense, nb, Hm, sb, sh, sm, sn, row_ptr, col_idx, partial, bits);
+  else
+    hipLaunchKernelGGL((pack_tiles_kernel<2, 1>), grid, dim3(256), 0, st, dense, nb, Hm, sb, sh, sm, sn, row_ptr, col_idx, partial, bits);
   return launch_status();
 }
 

@@ -34,6 +34,22 @@ def _prep(x):
     return x
 
 
+_workspaces = {}
+
+
+def _workspace(nbytes, device):
+    """Scratch memory for one call, kept per (device, stream) and reused by the next call on that stream:
+    the kernels need no particular contents on entry, and calls on one stream run one after the
+    other.  (Plans own their workspaces: they may be replayed from graphs on any stream.)"""
+    stream = torch.cuda.current_stream(device)
+    key = (device.index, stream.cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws, ctypes.c_void_p(stream.cuda_stream)
+
+
 def _like(x, dtype):
     """A result tensor laid out as the reference's torch.empty_like(x) lays it out (fa2_custom_mask.py:59,
     101-103): the dimension order of x by stride, without gaps.  For q, k, v sliced out of one packed
@@ -135,10 +151,10 @@ def _forward(q, k, v, lists, sm_scale, out_dtype, want_lse):
     o = _like(q, out_dtype)                                                     # :59
     lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device) if want_lse else None  # :70
     wsb = _ext.fwd_workspace(B, H, N, D, q.device)
-    ws = torch.empty(wsb, dtype=torch.uint8, device=q.device)
+    ws, stream = _workspace(wsb, q.device)
     common = (lists.Bm, lists.Hm, B, H, N, D, _ext.dtype_code(q.dtype), _ext.dtype_code(out_dtype), float(sm_scale),
               _ext.strides4(q), _ext.strides4(k), _ext.strides4(v), _ext.strides4(o),
-              ws.data_ptr(), wsb, _ext.current_stream(q.device))
+              ws.data_ptr(), wsb, stream)
     ptrs = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr() if want_lse else None,
             lists.row_ptr.data_ptr(), lists.col_idx.data_ptr())
     if _use_quads(lists, B, H, N, D):
@@ -199,7 +215,7 @@ def _backward(q, k, v, o, do, lse, lists, lists_t, sm_scale, out_dtype):
     q, k, v, o, do = _prep(q), _prep(k), _prep(v), _prep(o), _prep(do)
     dq, dk, dv = _like(q, out_dtype), _like(k, out_dtype), _like(v, out_dtype)   # :101-103
     wsb = _ext.bwd_workspace(B, H, N, D, q.device)
-    ws = torch.empty(wsb, dtype=torch.uint8, device=q.device)
+    ws, stream = _workspace(wsb, q.device)
     tensors = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(), lse.data_ptr(),
                dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
                lists.row_ptr.data_ptr(), lists.col_idx.data_ptr(), lists_t.row_ptr.data_ptr(),
@@ -208,7 +224,7 @@ def _backward(q, k, v, o, do, lse, lists, lists_t, sm_scale, out_dtype):
               _ext.dtype_code(q.dtype), _ext.dtype_code(out_dtype), float(sm_scale),
               _ext.strides4(q), _ext.strides4(k), _ext.strides4(v), _ext.strides4(o), _ext.strides4(do),
               _ext.strides4(dq), _ext.strides4(dk), _ext.strides4(dv),
-              ws.data_ptr(), wsb, _ext.current_stream(q.device))
+              ws.data_ptr(), wsb, stream)
     if lists.bits is None:
         rc = _ext.lib().bsattn_bwd(*tensors, *common)
     else:                                      # elementwise mask

@@ -124,12 +124,17 @@ def block_mask_to_lists(block, transpose=False, want_groups=False):
         raise ValueError("block mask must be square")
     dev = block.device
     rows = Bm * Hm * nb
-    row_ptr = torch.empty(rows + 1, dtype=torch.int32, device=dev)
-    col_idx = torch.empty(rows * nb, dtype=torch.int32, device=dev)
-    groups = torch.empty((rows, 5), dtype=torch.int32, device=dev) if want_groups else None
-    counts = torch.empty(2, dtype=torch.int32, device=dev)
+    # one allocation for everything the call writes: workspace | row_ptr | counts | col_idx | groups
     wsb = _ext.mask_lists_workspace(Bm, Hm, nb)
-    ws = torch.empty(wsb, dtype=torch.uint8, device=dev)
+    ws_ints = (wsb + 3) // 4
+    o_ptr = ws_ints
+    o_counts = o_ptr + rows + 1
+    o_cols = o_counts + 2
+    o_groups = o_cols + rows * nb
+    buf = torch.empty(o_groups + (rows * 5 if want_groups else 0), dtype=torch.int32, device=dev)
+    ws = buf[:ws_ints]
+    row_ptr, counts, col_idx = buf[o_ptr:o_counts], buf[o_counts:o_cols], buf[o_cols:o_groups]
+    groups = buf[o_groups:].view(rows, 5) if want_groups else None
     sb, sh, sm, sn = block.stride()
     if transpose:
         sm, sn = sn, sm

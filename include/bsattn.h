@@ -73,7 +73,8 @@ int bsattn_reduce_dense_mask(const uint8_t* dense, int Bm, int Hm, int N,
                              int64_t sb, int64_t sh, int64_t sm,
                              uint8_t* block_out, void* stream);
 
-/* Bytes of workspace bsattn_block_mask_to_lists needs for Bm*Hm*nb rows. */
+/* Bytes of workspace bsattn_block_mask_to_lists needs for Bm*Hm*nb rows (4-byte aligned; its contents
+ * on entry do not matter). */
 int bsattn_mask_lists_workspace(int Bm, int Hm, int nb, size_t* bytes);
 
 /* Block mask [Bm,Hm,nb,nb] (bool bytes, arbitrary element strides; pass the row/column
