@@ -23,10 +23,20 @@ KEEPS = [0.05, 0.1, 0.25, 0.5, 1.0]
 PEAK_F16_TFLOPS = 2500.0     # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0
 SEED = 1234 + 2
-# HBM-side bytes of one keep-1.0 forward launch, from two rocprofv3 --pmc runs (FETCH_SIZE x 2.0 and
-# WRITE_SIZE x 1.0 after scaling by the readings of a 256 MiB device copy): 204792 KiB fetched +
-# 11334 KiB written.
-TRAFFIC_BYTES_PER_LAUNCH = (204792 + 11334) * 1024
+PROFILE = os.path.join(ROOT, "profiles", "fwd_kernel_n17536_d64_fp16.md")
+
+
+def measured_traffic():
+    """HBM-side bytes of one keep-1.0 forward launch as the committed rocprofv3 summary states them (two
+    --pmc runs, FETCH_SIZE and WRITE_SIZE, scaled by the readings of a plain device copy): the line
+    `traffic_bytes_per_launch = <bytes>` of the summary, or None when the summary does not have it.
+    A counter run cannot happen inside this program; the summary names the command and the commit."""
+    import re
+    try:
+        m = re.search(r"traffic_bytes_per_launch\s*=\s*(\d+)", open(PROFILE).read())
+    except OSError:
+        return None
+    return int(m.group(1)) if m else None
 
 
 def tile_flops(kept):
@@ -45,30 +55,125 @@ def event_times(fn, iters, warmup, torch):
     return sorted(a.elapsed_time(b) for a, b in evs)       # ms
 
 
-def fwd_bwd_c5(torch, dev, fm, steps, warmup):
-    """HIP-event times of one forward call and one backward call at configs[4]."""
+def fwd_bwd_c5(torch, dev, fm, steps, warmup, check=True):
+    """HIP-event times of one forward call and one backward call at configs[4], in both output modes:
+    results typed bf16 like the inputs (what autograd hands back; P and dS rounded to bf16) and results in
+    fp32 (P and dS kept in fp16).  With check: relative L2 errors of O, dQ, dK, dV against the oracle
+    (numpy fp32 closed-form gradients) on two of the 32 heads."""
+    import numpy as np
     B, H, Nc, Dc = 2, 16, 8192, 128
     nbc = Nc // TILE
     g = torch.Generator().manual_seed(1238)
-    q, k, v, do = [torch.randn(B, H, Nc, Dc, generator=g).to(torch.bfloat16).to(dev) for _ in range(4)]
+    q, k, v, do = [torch.randn(B, H, Nc, Dc, generator=g).to(torch.bfloat16) for _ in range(4)]
     m = (torch.rand(1, 1, nbc, nbc, generator=g) < 0.25) | torch.eye(nbc, dtype=torch.bool)
-    m = torch.tril(m.reshape(nbc, nbc)).reshape(1, 1, nbc, nbc).to(dev)
-    lists = fm.block_mask_to_lists(m)
-    lists_t = fm.block_mask_to_lists(m, transpose=True)
+    m = torch.tril(m.reshape(nbc, nbc)).reshape(1, 1, nbc, nbc)
+    qd, kd, vd, dod, md = [x.to(dev) for x in (q, k, v, do, m)]
+    lists = fm.block_mask_to_lists(md)
+    lists_t = fm.block_mask_to_lists(md, transpose=True)
     tiles = int(lists.counts[1]) * B * H
     sc = 1.0 / Dc ** 0.5
-    fplan = fm.ForwardPlan(q, k, v, lists, sc)
-    o, lse = fplan.run()
-    bplan = fm.BackwardPlan(q, k, v, o, do, lse, lists, lists_t, sc)
-    tf = event_times(fplan.run, steps, warmup, torch)
-    tb = event_times(bplan.run, steps, warmup, torch)
-    mf, mb = tf[len(tf) // 2], tb[len(tb) // 2]
     ff, fb = tiles * 4.0 * TILE * TILE * Dc, tiles * 10.0 * TILE * TILE * Dc
-    return {"workload": "BASELINE configs[4]: fwd+bwd B=2 H=16 N=8192 D=128 bf16, block-causal keep 0.25 shared mask",
-            "kept_tiles": tiles, "fwd_ms": round(mf, 5), "fwd_tflops": round(ff / mf / 1e9, 1),
-            "bwd_ms": round(mb, 5), "bwd_tflops": round(fb / mb / 1e9, 1),
-            "frac_mfma_peak": {"fwd": round(ff / mf / 1e9 / PEAK_F16_TFLOPS, 4), "bwd": round(fb / mb / 1e9 / PEAK_F16_TFLOPS, 4)},
-            "note": "one bsattn_fwd call and one bsattn_bwd call (delta, dq and dkdv kernels), buffers allocated beforehand"}
+    out = {"workload": "BASELINE configs[4]: fwd+bwd B=2 H=16 N=8192 D=128 bf16, block-causal keep 0.25 shared mask",
+           "kept_tiles": tiles,
+           "note": "one bsattn_fwd call and one bsattn_bwd call (delta, dq and dkdv kernels), buffers allocated beforehand"}
+    ref = None
+    if check:
+        from oracle import bsattn_oracle as orc
+        heads = [(0, 0), (1, 15)]
+        ref = {}
+        for (b, h) in heads:
+            sl = (slice(b, b + 1), slice(h, h + 1))
+            f = lambda x: x[sl].float().numpy()
+            o_r = orc.naive_attention(f(q), f(k), f(v), m.numpy(), sc)
+            dq_r, dk_r, dv_r, _ = orc.attention_backward(f(q), f(k), f(v), m.numpy(), sc, f(do))
+            ref[(b, h)] = (o_r, dq_r, dk_r, dv_r)
+    for mode, odt in (("bf16_results", None), ("fp32_results", torch.float32)):
+        fplan = fm.ForwardPlan(qd, kd, vd, lists, sc, out_dtype=odt)
+        o, lse = fplan.run()
+        o_in = o if o.dtype == qd.dtype else o.to(qd.dtype)
+        bplan = fm.BackwardPlan(qd, kd, vd, o_in, dod, lse, lists, lists_t, sc, out_dtype=odt)
+        tf = event_times(fplan.run, steps, warmup, torch)
+        tb = event_times(bplan.run, steps, warmup, torch)
+        mf, mb = tf[len(tf) // 2], tb[len(tb) // 2]
+        rec = {"fwd_ms": round(mf, 5), "fwd_tflops": round(ff / mf / 1e9, 1), "bwd_ms": round(mb, 5),
+               "bwd_tflops": round(fb / mb / 1e9, 1),
+               "frac_mfma_peak": {"fwd": round(ff / mf / 1e9 / PEAK_F16_TFLOPS, 4), "bwd": round(fb / mb / 1e9 / PEAK_F16_TFLOPS, 4)}}
+        if ref is not None:
+            dq, dk, dv = bplan.run()
+            torch.cuda.synchronize()
+            worst = {"O": 0.0, "dQ": 0.0, "dK": 0.0, "dV": 0.0}
+            for (b, h), rs in ref.items():
+                for name, got, r in zip(("O", "dQ", "dK", "dV"), (o, dq, dk, dv), rs):
+                    gnp = got[b:b + 1, h:h + 1].float().cpu().numpy()
+                    worst[name] = max(worst[name], float(np.linalg.norm(gnp - r) / np.linalg.norm(r)))
+            rec["rel_l2_vs_oracle_2_heads"] = {kk: float("%.3e" % vv) for kk, vv in worst.items()}
+        out[mode] = rec
+        del fplan, bplan, o, lse
+    # the figures the earlier single-mode record carried, for the mode autograd uses
+    out.update({kk: out["bf16_results"][kk] for kk in ("fwd_ms", "fwd_tflops", "bwd_ms", "bwd_tflops", "frac_mfma_peak")})
+    return out
+
+
+def config_line(torch, dev, fm, name, N_, keeps, causal, seed, dense_mask_paths, reps=20):
+    """One BASELINE configuration at B=1 H=1 D=64 fp16: per kept ratio the kernel time (lists ready), the time
+    from a block mask on the device (lists built inside the call), optionally the time from a dense N x N
+    tile-constant bool mask (reduced to the block mask, or taken as an elementwise mask), and the parity of
+    sampled row blocks against the oracle."""
+    import numpy as np
+    from fa2_custom_mask import utils
+    from oracle import c_oracle
+    nb_ = N_ // TILE
+    g = torch.Generator().manual_seed(seed)
+    q, k, v = [torch.randn(1, 1, N_, D, generator=g).to(torch.float16) for _ in range(3)]
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    sc = 1.0 / D ** 0.5
+    out = {"workload": name, "keeps": {}}
+    for r in keeps:
+        m = (torch.rand(1, 1, nb_, nb_, generator=g) < r) | torch.eye(nb_, dtype=torch.bool)
+        if causal:
+            m = m & torch.tril(torch.ones(nb_, nb_, dtype=torch.bool))
+        md = m.to(dev)
+        lists = fm.block_mask_to_lists(md)
+        kept = int(lists.counts[1])
+        plan = fm.ForwardPlan(qd, kd, vd, lists, sc)
+        tk = event_times(plan.run, reps, 3, torch)
+
+        def from_block():
+            utils.lists_cache.clear()
+            return fm.flash_attention_custom_mask(qd, kd, vd, md, sc)
+        tb = event_times(from_block, reps, 3, torch)
+        med = tk[len(tk) // 2]
+        rec = {"kept_tiles": kept, "kernel_ms": round(med, 5),
+               "tflops_on_kept_tiles": round(tile_flops(kept) / med / 1e9, 1),
+               "frac_mfma_peak": round(tile_flops(kept) / med / 1e9 / PEAK_F16_TFLOPS, 4),
+               "from_block_mask_ms": round(tb[len(tb) // 2], 5)}
+        if dense_mask_paths:
+            dense = md.repeat_interleave(TILE, 2).repeat_interleave(TILE, 3).contiguous()
+
+            def from_dense_reduced():
+                utils.lists_cache.clear()
+                return fm.flash_attention_custom_mask(qd, kd, vd, fm.reduce_dense_mask(dense), sc)
+
+            def from_dense_elementwise():
+                utils.lists_cache.clear()
+                return fm.flash_attention_custom_mask(qd, kd, vd, dense, sc)
+            t1 = event_times(from_dense_reduced, reps, 3, torch)
+            t2 = event_times(from_dense_elementwise, reps, 3, torch)
+            rec["from_dense_mask_reduced_ms"] = round(t1[len(t1) // 2], 5)
+            rec["from_dense_mask_elementwise_ms"] = round(t2[len(t2) // 2], 5)
+            del dense
+        o = plan.run()[0]
+        torch.cuda.synchronize()
+        worst = 0.0
+        for rb in sorted({0, nb_ // 2, nb_ - 1}):
+            o_ref, _ = c_oracle.naive_fwd(q.float().numpy(), k.float().numpy(), v.float().numpy(), m.numpy(), sc,
+                                          rb * TILE, rb * TILE + TILE)
+            worst = max(worst, float(np.abs(o[0, 0, rb * TILE:(rb + 1) * TILE].float().cpu().numpy()
+                                            - o_ref[0, 0, rb * TILE:(rb + 1) * TILE]).max()))
+        rec["max_abs_vs_oracle_sampled_rows"] = worst
+        out["keeps"][str(r)] = rec
+        del plan, lists
+    return out
 
 
 def elementwise_case(torch, dev, fm, q, k, v, sm_scale):
@@ -204,7 +309,7 @@ def main():
         print(json.dumps(reorder_case(torch, dev, fm)))
         return
     if args.fwd_bwd:
-        print(json.dumps(fwd_bwd_c5(torch, dev, fm, min(args.steps, 50), min(args.warmup, 5))))
+        print(json.dumps(fwd_bwd_c5(torch, dev, fm, min(args.steps, 50), min(args.warmup, 5), check=not args.no_cpu)))
         return
     g = torch.Generator().manual_seed(SEED)
     q, k, v = [torch.randn(1, 1, N, D, generator=g).to(torch.float16) for _ in range(3)]
@@ -294,11 +399,18 @@ def main():
                             "block_mask_ms": round(ts_b[len(ts_b) // 2], 5)},
         "parity_max_abs_vs_oracle": parity,
         "data_dependence": data_dependence,
-        "fwd_bwd_configs4": fwd_bwd_c5(torch, dev, fm, 20, 3),
+        "configs0": config_line(torch, dev, fm, "BASELINE configs[0]: fwd B=1 H=1 N=1024 D=64 fp16, keep 0.5 + diagonal",
+                                1024, [0.5], False, 1234, False),
+        "configs1": config_line(torch, dev, fm, "BASELINE configs[1]: fwd B=1 H=1 N=6400 D=64 fp16, keep 0.1 / 1.0, "
+                                "preprocessing from a dense tile-constant N x N bool mask included",
+                                6400, [0.1, 1.0], False, 1235, True),
+        "configs3": config_line(torch, dev, fm, "BASELINE configs[3]: fwd B=1 H=1 N=32000 D=64 fp16, block-causal x "
+                                "Bernoulli keep 0.1 / 1.0 + diagonal", 32000, [0.1, 1.0], True, 1237, False, reps=10),
+        "fwd_bwd_configs4": fwd_bwd_c5(torch, dev, fm, 20, 3, check=not args.no_cpu),
         "elementwise_mask": elementwise_case(torch, dev, fm, qd, kd, vd, sm_scale),
         "token_reorder": reorder_case(torch, dev, fm),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": TRAFFIC_BYTES_PER_LAUNCH,
+                     "frac": round(achieved / PEAK_F16_TFLOPS, 4), "traffic": measured_traffic(),
                      "kernel": "fwd_kernel<64, 0, false, false, true> (fp16, contiguous rows, one bsattn_fwd call)",
                      "algorithmic_flops_per_launch": tile_flops(kept[1.0])},
     }

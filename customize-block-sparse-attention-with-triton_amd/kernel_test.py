@@ -3,7 +3,7 @@
 reference: sequence length, kept ratio, `flash_attention_custom_mask` time including mask
 preprocessing, naive matmul+softmax time, speed-up), for this package on an MI355X.
 
-    python kernel_test.py [--seq-len 6400 17536 32000] [--ratio 0.1 1.0] [--heads 1] [--dim 64]
+    python kernel_test.py [--seq-len 6400 17536 32000] [--ratio 0.1 1.0] [--heads 8] [--dim 64]
 
 Like the reference's kernel-test.py (:12-19) the inputs are N(0,1) fp16, the block mask is
 Bernoulli(ratio), and the naive path expands the mask to N x N; unlike it the runs are seeded,
@@ -34,17 +34,17 @@ def timed(fn, reps):
     return sorted(ts)[len(ts) // 2]
 
 
-def main():
+def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--seq-len", type=int, nargs="+", default=[6400, 17536, 32000])
     ap.add_argument("--ratio", type=float, nargs="+", default=[0.1, 1.0])
     ap.add_argument("--batch", type=int, default=1)
-    ap.add_argument("--heads", type=int, default=1)
+    ap.add_argument("--heads", type=int, default=8)          # kernel-test.py:7
     ap.add_argument("--dim", type=int, default=64)
     ap.add_argument("--reps", type=int, default=5)
     ap.add_argument("--naive-limit-gb", type=float, default=40.0,
                     help="skip the naive path when its fp16 N x N scores exceed this many GB")
-    args = ap.parse_args()
+    args = ap.parse_args(argv)
     dev = torch.device("cuda:0")
     print("| [seq_len, dim] | ratio | custom mask incl. preprocessing (s) | cached lists (s) | naive matmul+softmax (s) | speed-up | max abs diff |")
     print("|---|---|---|---|---|---|---|")
