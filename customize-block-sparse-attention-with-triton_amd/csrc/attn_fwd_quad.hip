@@ -70,6 +70,16 @@ __device__ __forceinline__ int wave_inclusive_sum(int v, int lane) {
   return v;
 }
 
+// Measurement build only (-DQUAD_TIMELINE, never the library's): every wavefront group writes the 100 MHz
+// wall clock at four points (entry, first round, last round done, row blocks finished) to a buffer whose
+// address the launcher takes from the environment variable BSATTN_QUAD_TIMELINE.
+#ifdef QUAD_TIMELINE
+#define QUAD_WALL(i) do { if (prm.part_o != nullptr && (threadIdx.x & 255) == 0) \
+    reinterpret_cast<long long*>(prm.part_o)[(blockIdx.x * 2 + (threadIdx.x >> 8)) * 4 + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#else
+#define QUAD_WALL(i) do {} while (0)
+#endif
+
 template <int DT, bool CONTIG>
 __global__ __launch_bounds__(512, 1)
 void fwd_quad_kernel(const FwdParams prm) {
@@ -81,6 +91,7 @@ void fwd_quad_kernel(const FwdParams prm) {
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
 
   const int lane = threadIdx.x & 63;
+  QUAD_WALL(0);
   const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int grp = w >> 2, r = w & 3;     // wavefronts r and r + 4 share a SIMD
   const int ln = lane & 31, g = lane >> 5;
@@ -534,6 +545,7 @@ void fwd_quad_kernel(const FwdParams prm) {
   copies_ahead(n > 1);
   sync();                                 // the first K tile is complete
   if (grp == 1) sync();                   // the second group runs one phase behind the first
+  QUAD_WALL(1);
 
   // =========================== segments ===========================
   for (;;) {
@@ -546,9 +558,16 @@ void fwd_quad_kernel(const FwdParams prm) {
       const bool mine = (entry >> (16 + r)) & 1;
       const unsigned char* lds_k = tiles + kt * C::TILE_BYTES;
       uintx4 vfr[4][DB], kfr[2][KS];
+#ifdef QUAD_PRIO_M
+      __builtin_amdgcn_s_setprio(QUAD_PRIO_M);
+#endif
       // (read whether needed or not: a wavefront that sits the tile out ignores what it gets)
       read_v(tiles + (3 + ((t - 1) & 1)) * C::TILE_BYTES, vfr);
       read_k(lds_k, kfr);
+      // all sixteen reads are on their way before the first MFMA waits for one (left to itself the compiler
+      // reads the V fragments one at a time into one register group, each read a full LDS round trip in
+      // front of two MFMAs)
+      __builtin_amdgcn_sched_barrier(0);
       if (p_live) { second_product(vfr); p_live = false; }
       // list entries of the next round (picked up in the vector phase)
       int raw_entry = 0, raw_next = 0;
@@ -562,6 +581,9 @@ void fwd_quad_kernel(const FwdParams prm) {
         first_product(kfr, sa0, sa1, sb0, sb1);
         had_tiles = true;
         sync();
+#ifdef QUAD_PRIO_M
+        __builtin_amdgcn_s_setprio(QUAD_PRIO_V);
+#endif
         numerators(lds_k, sa0, sa1, sb0, sb1, pf);
         p_live = true;
       } else {
@@ -591,7 +613,9 @@ void fwd_quad_kernel(const FwdParams prm) {
       read_v(tiles + (3 + ((t - 1) & 1)) * C::TILE_BYTES, vfr);
       second_product(vfr);
     }
+    if (!more) QUAD_WALL(2);
     finish_rowblock(seg, had_tiles);
+    if (!more) QUAD_WALL(3);
     if (!more) return;
     __builtin_amdgcn_s_waitcnt(0x0F70);   // (Q, and whatever finishing the row block left in flight)
     sync();

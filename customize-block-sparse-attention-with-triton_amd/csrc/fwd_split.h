@@ -31,6 +31,11 @@ __device__ __forceinline__ HeadSplit head_split(Ptr rp, int nb, int P, int min_t
   const int want = (s.T + min_tiles - 1) / min_tiles;   // no range shorter than about min_tiles
   s.Peff = want < P ? want : P;
   s.fast = fast < 0 ? 0 : (fast < s.Peff ? fast : s.Peff);
+#ifndef EQUAL_SPLIT_BELOW
+#define EQUAL_SPLIT_BELOW 48
+#endif
+  // short ranges are a matter of latency, which both workgroups of a compute unit see alike: equal shares
+  if ((int64_t)s.T < (int64_t)EQUAL_SPLIT_BELOW * s.Peff) s.fast = 0;
   s.ctot = split_cum(s, s.Peff);
   return s;
 }
