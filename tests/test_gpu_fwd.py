@@ -302,3 +302,30 @@ def test_cached_lists_on_another_stream(dev):
     side.synchronize()
     torch.cuda.synchronize()
     assert errors(o1, o_ref)[1] <= RELL2 and errors(o2, o_ref)[1] <= RELL2
+
+
+@pytest.mark.parametrize("dtype,out_fp32", [(torch.float16, False), (torch.bfloat16, False), (torch.bfloat16, True)])
+def test_large_magnitudes(dev, dtype, out_fp32):
+    """Inputs far from N(0,1): scores with a standard deviation of 23 (a nearly one-hot softmax whose reference
+    exponent moves by hundreds between tiles) and values of the order of 1e3.  The kernels fold the scale
+    into a 16-bit Q, feed exponents through an extra contraction slice and, for bf16 inputs with fp32
+    results, convert V to fp16: all of that must hold up, relative to the size of the values."""
+    import fa2_custom_mask as fm
+    B, H, N, D = 1, 2, 1024, 64
+    g = torch.Generator().manual_seed(77)
+    q = (torch.randn(B, H, N, D, generator=g) * 4.0).to(dtype)
+    k = (torch.randn(B, H, N, D, generator=g) * 4.0).to(dtype)
+    v = (torch.randn(B, H, N, D, generator=g) * 1000.0).to(dtype)
+    mask = uniform_block_mask(1, 1, 16, 0.5, 12)
+    sc = 0.18
+    o_ref, lse_ref = orc.naive_attention(f32(q), f32(k), f32(v), mask.numpy(), sc, return_lse=True)
+    o, lse = fm.flash_attention_custom_mask_lse(q.to(dev), k.to(dev), v.to(dev), mask.to(dev), sc, out_fp32=out_fp32)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(o).all())
+    ma, rl = errors(o, o_ref)
+    scale = float(np.abs(o_ref).max())
+    print("%s fp32out=%s: max-abs %.3e of %.3e, rel-L2 %.3e" % (dtype, out_fp32, ma, scale, rl))
+    # the bars of the forward tests, relative to the size of the result
+    assert ma <= (2e-2 if dtype == torch.float16 else 3e-2) * max(1.0, scale / 4.0)
+    assert rl <= (1e-3 if dtype == torch.float16 or out_fp32 else 3e-3) * 1.5
+    assert np.abs(lse.cpu().numpy() - lse_ref).max() <= 2e-3 * max(1.0, float(np.abs(lse_ref).max()) / 8.0)
