@@ -375,7 +375,8 @@ def main():
     ts = event_times(lambda: fm.block_mask_to_lists(fm.reduce_dense_mask(dense_mask)), 20, 3, torch)
     pre_ms = ts[len(ts) // 2]
     pre_bytes = float(N) * N + 4.0 * (kept[0.1] + 5 * NB)
-    ts_b = event_times(lambda: fm.block_mask_to_lists(masks[0.1].to(dev)), 20, 3, torch)
+    block_dev = masks[0.1].to(dev)
+    ts_b = event_times(lambda: fm.block_mask_to_lists(block_dev), 20, 3, torch)
     del dense_mask
 
     # ---- parity spot check against the CPU oracle (first 2 row blocks, keep 0.1) ----
