@@ -79,6 +79,30 @@ int bsattn_pack_mask_tiles(const uint8_t* dense, int Bm, int Hm, int N, int64_t 
                            (unsigned long long*)tile_bits, (hipStream_t)stream);
 }
 
+int bsattn_reduce_pack_dense_mask(const uint8_t* dense, int Bm, int Hm, int N, int64_t sb, int64_t sh, int64_t sm,
+                                  uint8_t* block_out, uint8_t* grid_partial, uint64_t* grid_bits, void* stream) {
+  if (dense == nullptr || block_out == nullptr || grid_partial == nullptr || grid_bits == nullptr) return BSATTN_ERR_NULL;
+  if (Bm <= 0 || Hm <= 0 || N <= 0 || N % BSATTN_TILE != 0) return BSATTN_ERR_SHAPE;
+  if ((int64_t)Bm * Hm > 65535) return BSATTN_ERR_RANGE;
+  if ((sm % 16) != 0 || (sb % 16) != 0 || (sh % 16) != 0 || ((uintptr_t)dense & 15) != 0 || ((uintptr_t)grid_bits & 7) != 0)
+    return BSATTN_ERR_STRIDE;
+  return launch_reduce_pack(dense, Bm, Hm, N, sb, sh, sm, block_out, grid_partial, (unsigned long long*)grid_bits,
+                            (hipStream_t)stream);
+}
+
+int bsattn_gather_mask_tiles(const uint8_t* grid_partial, const uint64_t* grid_bits, int Bm, int Hm, int nb,
+                             int transposed, const int32_t* row_ptr, const int32_t* col_idx, uint8_t* tile_partial,
+                             uint64_t* tile_bits, void* stream) {
+  if (grid_partial == nullptr || grid_bits == nullptr || row_ptr == nullptr || col_idx == nullptr ||
+      tile_partial == nullptr || tile_bits == nullptr)
+    return BSATTN_ERR_NULL;
+  if (Bm <= 0 || Hm <= 0 || nb <= 0) return BSATTN_ERR_SHAPE;
+  if ((int64_t)Bm * Hm > 65535 || (int64_t)Bm * Hm * nb * nb > 0x7fffffffLL) return BSATTN_ERR_RANGE;
+  if ((((uintptr_t)grid_bits | (uintptr_t)tile_bits) & 7) != 0) return BSATTN_ERR_STRIDE;
+  return launch_gather_tiles(grid_partial, (const unsigned long long*)grid_bits, Bm, Hm, nb, transposed != 0, row_ptr, col_idx,
+                             tile_partial, (unsigned long long*)tile_bits, (hipStream_t)stream);
+}
+
 int bsattn_tail_mask_tiles(int Bm, int Hm, int nb, int valid_last, int transposed, const int32_t* row_ptr,
                            const int32_t* col_idx, uint8_t* tile_partial, uint64_t* tile_bits, void* stream) {
   if (row_ptr == nullptr || col_idx == nullptr || tile_partial == nullptr || tile_bits == nullptr) return BSATTN_ERR_NULL;

@@ -20,6 +20,11 @@ int launch_quad_lists(const int32_t* row_ptr, const int32_t* col_idx, int Bm, in
                       int32_t* quad_list, int32_t* stats, hipStream_t st);
 int launch_tail_tiles(int Bm, int Hm, int nb, int valid, int transpose, const int32_t* row_ptr,
                       const int32_t* col_idx, uint8_t* partial, unsigned long long* bits, hipStream_t st);
+int launch_reduce_pack(const uint8_t* dense, int Bm, int Hm, int N, int64_t sb, int64_t sh, int64_t sm,
+                       uint8_t* block_out, uint8_t* grid_partial, unsigned long long* grid_bits, hipStream_t st);
+int launch_gather_tiles(const uint8_t* grid_partial, const unsigned long long* grid_bits, int Bm, int Hm, int nb,
+                        int transposed, const int32_t* row_ptr, const int32_t* col_idx, uint8_t* partial,
+                        unsigned long long* bits, hipStream_t st);
 int launch_pack_tiles(const uint8_t* dense, int Bm, int Hm, int nb, int64_t sb, int64_t sh, int64_t sm,
                       int64_t sn, const int32_t* row_ptr, const int32_t* col_idx, uint8_t* partial,
                       unsigned long long* bits, hipStream_t st);

@@ -301,6 +301,116 @@ __global__ __launch_bounds__(256) void pack_tiles_kernel(const uint8_t* __restri
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Elementwise masks in one pass over the mask: block mask, "partly set" flags and the packed words of every
+// tile that has a set element, all indexed by the tile's position in the grid ((mask head * nb + row block) * nb
+// + column block), since the lists do not exist yet.  gather_tiles_kernel then moves the words of the kept
+// tiles to their list positions, for the row lists as they are and for the column lists transposed, so the
+// mask itself (Bm Hm N^2 bytes) is read once, in whole rows, whatever is made of it afterwards.
+// As reduce_dense_kernel, one wavefront owns 64 rows x 1024 columns (16 tiles): a lane reads its 16-byte
+// column slice of every row (16 rows in flight), turns it into 16 bits, the four lanes of a tile put theirs
+// together, and the words wait in LDS until the 64 rows are through; then lane l holds the word of row l of
+// each tile and the wavefront writes 512 contiguous bytes per tile.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void reduce_pack_kernel(const uint8_t* __restrict__ dense, int N, int nb, int H,
+                                                          int64_t sb, int64_t sh, int64_t sm,
+                                                          uint8_t* __restrict__ block, uint8_t* __restrict__ grid_partial,
+                                                          unsigned long long* __restrict__ grid_bits) {
+  __shared__ unsigned long long stage[4][16][64];      // [wavefront][tile][row]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int rb = blockIdx.x;
+  const int col0 = (blockIdx.y * 4 + wave) * 1024;
+  if (col0 >= N) return;
+  const int bh = blockIdx.z;
+  const int b = bh / H, h = bh % H;
+  const int col = col0 + lane * 16;
+  const bool in = col < N;
+  const uint8_t* p = dense + b * sb + h * sh + (int64_t)rb * 64 * sm + (in ? col : 0);
+  const int j = lane >> 2, chunk = lane & 3;
+  unsigned long long (*my)[64] = stage[wave];
+#pragma unroll 1
+  for (int r0 = 0; r0 < 64; r0 += 16) {
+    u32x4 d[16];
+#pragma unroll
+    for (int it = 0; it < 16; ++it) d[it] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + (r0 + it) * sm));
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+      const unsigned hbits = in ? bools16(d[it]) : 0u;
+      const unsigned h0 = __builtin_amdgcn_mov_dpp(hbits, 0x00, 0xf, 0xf, true), h1 = __builtin_amdgcn_mov_dpp(hbits, 0x55, 0xf, 0xf, true);
+      const unsigned h2 = __builtin_amdgcn_mov_dpp(hbits, 0xaa, 0xf, 0xf, true), h3 = __builtin_amdgcn_mov_dpp(hbits, 0xff, 0xf, 0xf, true);
+      const unsigned long long x = (unsigned long long)(h0 | (h1 << 16)) | ((unsigned long long)(h2 | (h3 << 16)) << 32);
+      if (chunk == 0) my[j][r0 + it] = x;
+    }
+  }
+  // (the LDS operations of one wavefront complete in order: the reads below see the writes above)
+  const int t0 = col0 >> 6;
+#pragma unroll 1
+  for (int jj = 0; jj < 16; ++jj) {
+    const int t = t0 + jj;
+    if (t >= nb) break;
+    const unsigned long long word = my[jj][lane];
+    const bool any = __ballot(word != 0ull) != 0ull;
+    const bool full = __ballot(word == ~0ull) == ~0ull;
+    const int64_t tile = ((int64_t)bh * nb + rb) * nb + t;
+    if (any) grid_bits[tile * 64 + lane] = word;        // (tiles without a set element are never looked at)
+    if (lane == 0) { block[tile] = any ? 1 : 0; grid_partial[tile] = any && !full ? 1 : 0; }
+  }
+}
+
+// Words of the kept tiles from their grid positions to their list positions.  TRANSPOSE: the lists are the column
+// lists (list row = column block a, entries = row blocks), and the words are wanted per key with one bit per
+// query: the 64 x 64 bit matrix is transposed with one ballot per word.  One workgroup of four wavefronts per
+// GATHER_SPLIT-th of a list row, a wavefront per entry.
+constexpr int GATHER_SPLIT = 4;
+template <bool TRANSPOSE>
+__global__ __launch_bounds__(256) void gather_tiles_kernel(const uint8_t* __restrict__ grid_partial,
+                                                           const unsigned long long* __restrict__ grid_bits, int nb,
+                                                           const int32_t* __restrict__ row_ptr,
+                                                           const int32_t* __restrict__ col_idx,
+                                                           uint8_t* __restrict__ partial,
+                                                           unsigned long long* __restrict__ bits) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int a = blockIdx.x / GATHER_SPLIT, sub = blockIdx.x % GATHER_SPLIT, mh = blockIdx.y;
+  const int32_t* rp = row_ptr + (int64_t)mh * nb;
+  const int t0 = rp[a], t1 = rp[a + 1];
+  for (int t = t0 + sub * 4 + wave; t < t1; t += 4 * GATHER_SPLIT) {
+    const int other = col_idx[t];
+    const int64_t tile = TRANSPOSE ? ((int64_t)mh * nb + other) * nb + a : ((int64_t)mh * nb + a) * nb + other;
+    unsigned long long word = grid_bits[tile * 64 + lane];
+    if constexpr (TRANSPOSE) {
+      unsigned long long out = 0ull;
+#pragma unroll 8
+      for (int r = 0; r < 64; ++r) {
+        const unsigned long long bal = __ballot((word >> r) & 1ull);
+        if (lane == r) out = bal;
+      }
+      word = out;
+    }
+    bits[(int64_t)t * 64 + lane] = word;
+    if (lane == 0) partial[t] = grid_partial[tile];
+  }
+}
+
+int launch_reduce_pack(const uint8_t* dense, int Bm, int Hm, int N, int64_t sb, int64_t sh, int64_t sm,
+                       uint8_t* block_out, uint8_t* grid_partial, unsigned long long* grid_bits, hipStream_t st) {
+  const int nb = N / 64;
+  dim3 grid(nb, (N + 4095) / 4096, Bm * Hm);
+  hipLaunchKernelGGL(reduce_pack_kernel, grid, dim3(256), 0, st, dense, N, nb, Hm, sb, sh, sm, block_out, grid_partial,
+                     grid_bits);
+  return launch_status();
+}
+
+int launch_gather_tiles(const uint8_t* grid_partial, const unsigned long long* grid_bits, int Bm, int Hm, int nb,
+                        int transposed, const int32_t* row_ptr, const int32_t* col_idx, uint8_t* partial,
+                        unsigned long long* bits, hipStream_t st) {
+  const dim3 grid(nb * GATHER_SPLIT, Bm * Hm);
+  if (transposed)
+    hipLaunchKernelGGL(gather_tiles_kernel<true>, grid, dim3(256), 0, st, grid_partial, grid_bits, nb, row_ptr, col_idx, partial, bits);
+  else
+    hipLaunchKernelGGL(gather_tiles_kernel<false>, grid, dim3(256), 0, st, grid_partial, grid_bits, nb, row_ptr, col_idx, partial, bits);
+  return launch_status();
+}
+
 int launch_reduce_dense_mask(const uint8_t* dense, int Bm, int Hm, int N, int64_t sb, int64_t sh,
                              int64_t sm, uint8_t* block_out, hipStream_t st) {
   const int nb = N / 64;

@@ -26,6 +26,8 @@ _SIGNATURES = {
     "bsattn_block_mask_to_lists": ([_p, _i, _i, _i, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p,
                                     ctypes.c_size_t, _p], _i),
     "bsattn_pack_mask_tiles": ([_p, _i, _i, _i, _i64, _i64, _i64, _i64, _p, _p, _p, _p, _p], _i),
+    "bsattn_reduce_pack_dense_mask": ([_p, _i, _i, _i, _i64, _i64, _i64, _p, _p, _p, _p], _i),
+    "bsattn_gather_mask_tiles": ([_p, _p, _i, _i, _i, _i, _p, _p, _p, _p, _p], _i),
     "bsattn_tail_mask_tiles": ([_i, _i, _i, _i, _i, _p, _p, _p, _p, _p], _i),
     "bsattn_fwd_workspace": ([_i, _i, _i, _i, ctypes.POINTER(ctypes.c_size_t)], _i),
     "bsattn_fwd": ([_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f,

@@ -274,7 +274,8 @@ class _attention(torch.autograd.Function):
         B, H, N, D = _check_qkv(q, k, v, mask)
         if mask is None:
             mask = _dense_mask(q.device, num_tiles(N))
-        lists = mask_to_lists(mask, N)                                       # :48
+        # (a backward will ask for the column lists too when a gradient is wanted)
+        lists = mask_to_lists(mask, N, both=any(ctx.needs_input_grad[:3]))   # :48
         out_dtype = torch.float32 if out_fp32 else q.dtype
         q, k, v = _padded(q, N, D), _padded(k, N, D), _padded(v, N, D)
         o, lse = _forward(q, k, v, lists, sm_scale, out_dtype, True)
@@ -329,7 +330,7 @@ def attention_forward_backward(q, k, v, mask, sm_scale, do, out_fp32=False):
     B, H, N, D = _check_qkv(q, k, v, mask)
     if mask is None:
         mask = _dense_mask(q.device, num_tiles(N))
-    lists = mask_to_lists(mask, N)
+    lists = mask_to_lists(mask, N, both=True)
     lists_t = mask_to_lists(mask, N, transpose=True)
     out_dtype = torch.float32 if out_fp32 else q.dtype
     q, k, v = _padded(q, N, D), _padded(k, N, D), _padded(v, N, D)

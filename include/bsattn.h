@@ -125,6 +125,24 @@ int bsattn_pack_mask_tiles(const uint8_t* dense, int Bm, int Hm, int N, int64_t 
                            int64_t sm, int64_t sn, const int32_t* row_ptr, const int32_t* col_idx,
                            uint8_t* tile_partial, uint64_t* tile_bits, void* stream);
 
+/* The same words in one pass over the mask, for callers that start from the elementwise mask itself: the
+ * block mask (as bsattn_reduce_dense_mask gives it), and for every tile of the grid that has a set element
+ * its "partly set" flag and its 64 words, at the tile's grid position
+ * g = (mask head * nb + row block) * nb + column block: grid_partial[g], grid_bits[64 g + r] (tiles without
+ * a set element get grid_partial = 0 and their words are left unwritten).  dense: innermost stride 1, the
+ * other strides multiples of 16 and a 16-byte aligned base; grid_partial: Bm*Hm*nb*nb bytes, grid_bits: 64
+ * times as many 64-bit words.  bsattn_gather_mask_tiles then moves the words of the kept tiles to their
+ * list positions (the format bsattn_fwd_elementwise / bsattn_bwd_elementwise take): with the row lists and
+ * transposed = 0 as they are, with the column lists (bsattn_block_mask_to_lists with the block mask's row
+ * and column strides swapped) and transposed = 1 as the per-key words of the dK/dV pass.  The mask is read
+ * once for all of it.  Same semantics as bsattn_pack_mask_tiles (kernel-test.py:38). */
+int bsattn_reduce_pack_dense_mask(const uint8_t* dense, int Bm, int Hm, int N, int64_t sb, int64_t sh,
+                                  int64_t sm, uint8_t* block_out, uint8_t* grid_partial,
+                                  uint64_t* grid_bits, void* stream);
+int bsattn_gather_mask_tiles(const uint8_t* grid_partial, const uint64_t* grid_bits, int Bm, int Hm,
+                             int nb, int transposed, const int32_t* row_ptr, const int32_t* col_idx,
+                             uint8_t* tile_partial, uint64_t* tile_bits, void* stream);
+
 /* Sequence lengths N that are not a multiple of 64 (unsupported by the reference, whose block
  * pointers assume whole tiles: fa2_custom_mask/fa2_fwd.py:137-172): the caller pads q, k, v
  * with zero rows to nb*64 tokens and masks the padding keys through the elementwise entry

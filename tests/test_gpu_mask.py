@@ -115,3 +115,33 @@ def test_pack_mask_tiles_bit_exact(dev, transpose):
             assert T == len(p_ref)
             assert np.array_equal(partial[:T].cpu().numpy(), p_ref)
             assert np.array_equal(bits[:T].cpu().numpy().view(np.uint64), w_ref)
+
+
+@pytest.mark.parametrize("transpose", [False, True])
+def test_one_pass_words_bit_exact(dev, transpose):
+    """The same words made in one pass over the mask (block mask + grid-ordered words, then gathered into list
+    order): bit-exact against the oracle and against the two-pass route, for both list orientations, several
+    mask heads, sizes that are not a multiple of 1024 columns, and a non-contiguous view."""
+    import fa2_custom_mask as fm
+    from fa2_custom_mask import utils
+    g = torch.Generator().manual_seed(18)
+    for shape, p in (((1, 1, 256, 256), 0.5), ((2, 3, 192, 192), 0.05), ((1, 2, 1344, 1344), 0.9), ((1, 1, 2112, 2112), 0.02)):
+        dense = torch.rand(shape, generator=g) < p
+        dense[0, 0, :64, :64] = True
+        dense[0, -1, 64:128, :] = False
+        variants = [dense.to(dev)]
+        big = torch.zeros(shape[:3] + (shape[3] + 64,), dtype=torch.bool)
+        big[..., :shape[3]] = dense
+        variants.append(big.to(dev)[..., :shape[3]])                 # padded rows: not contiguous
+        for md in variants:
+            block, gp, gb = utils.reduce_pack_dense_mask(md)
+            assert np.array_equal(block.cpu().numpy(), orc.reduce_dense_mask(dense.numpy()))
+            lists = fm.block_mask_to_lists(block, transpose=transpose)
+            partial, bits = utils.gather_mask_tiles(gp, gb, lists, transpose=transpose)
+            T = int(lists.counts[1])
+            p_ref, w_ref = orc.pack_mask_tiles(dense.numpy(), transpose)
+            assert T == len(p_ref)
+            assert np.array_equal(partial[:T].cpu().numpy(), p_ref)
+            assert np.array_equal(bits[:T].cpu().numpy().view(np.uint64), w_ref)
+            p2, b2 = utils.pack_mask_tiles(md, lists, transpose=transpose)
+            assert torch.equal(p2[:T], partial[:T]) and torch.equal(b2[:T], bits[:T])
