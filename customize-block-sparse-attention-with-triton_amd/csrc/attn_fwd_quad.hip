@@ -558,9 +558,6 @@ void fwd_quad_kernel(const FwdParams prm) {
       const bool mine = (entry >> (16 + r)) & 1;
       const unsigned char* lds_k = tiles + kt * C::TILE_BYTES;
       uintx4 vfr[4][DB], kfr[2][KS];
-#ifdef QUAD_PRIO_M
-      __builtin_amdgcn_s_setprio(QUAD_PRIO_M);
-#endif
       // (read whether needed or not: a wavefront that sits the tile out ignores what it gets)
       read_v(tiles + (3 + ((t - 1) & 1)) * C::TILE_BYTES, vfr);
       read_k(lds_k, kfr);
@@ -581,9 +578,6 @@ void fwd_quad_kernel(const FwdParams prm) {
         first_product(kfr, sa0, sa1, sb0, sb1);
         had_tiles = true;
         sync();
-#ifdef QUAD_PRIO_M
-        __builtin_amdgcn_s_setprio(QUAD_PRIO_V);
-#endif
         numerators(lds_k, sa0, sa1, sb0, sb1, pf);
         p_live = true;
       } else {
