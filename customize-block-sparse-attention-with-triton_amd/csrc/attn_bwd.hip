@@ -606,6 +606,251 @@ __global__ __launch_bounds__(128, (QB == 1 && D == 64) ? 2 : 1) void dkdv_kernel
 }
 
 // ---------------------------------------------------------------------------------------
+// dK, dV at D = 128 with block masks: workgroup = column block n, four wavefronts (one per SIMD).
+// Wavefront (kh, dh) owns keys 64n + 32kh + ln and the columns 64dh .. 64dh + 63 of their dK and dV rows: half
+// the accumulators of dkdv_kernel's wavefront, which, with K, V, dK and dV of its keys in 192 of 512
+// registers, runs alone on its SIMD and leaves the matrix cores idle two thirds of the time.  Here a wavefront
+// stays within 256 registers and two workgroups share a compute unit (two wavefronts per SIMD).
+// The first products (S, dP) contract over the whole head dimension, so the two wavefronts of a key half share
+// them by query block: wavefront dh computes S and dP of queries 32dh .. 32dh + 31, turns them into P and dS,
+// and hands both, packed as the operand fragments of the second products, to its partner through LDS (4 KB
+// each way, one barrier).  Every wavefront then runs the second products of both query blocks on its columns,
+// its own block first, while the partner's P and dS are on their way.
+// The per-query terms (- lse in the exponent, - delta beside dP) enter through one extra contraction slice each,
+// ones x the term in three 16-bit pieces, as the forward does with its reference exponent: no vector
+// instruction per element, and the row statistics need no place in LDS: a lane reads the two values of its
+// query from memory a step ahead.  (Two stages of a Q and a dO tile, 64 KB, + 16 KB of exchange are exactly half
+// the 160 KB of a compute unit: two workgroups per compute unit, two wavefronts per SIMD.)
+// ---------------------------------------------------------------------------------------
+template <int NWV, int D, int ROWS>
+__device__ __forceinline__ void part_tile_load_async(const unsigned short* tile, int64_t stride, int wv, int lane,
+                                                     unsigned lds_addr) {
+  constexpr int CPR = D / 8, PER_WAVE = ROWS * CPR / (64 * NWV);
+#pragma unroll
+  for (int jj = 0; jj < PER_WAVE; ++jj) {
+    const int j = wv * PER_WAVE + jj;
+    const int c = j * 64 + lane, row = c / CPR, ch = c % CPR;
+    const unsigned off = 2u * (unsigned)(row * (int)stride + ((ch ^ u_swz<D>(row)) * 8));
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_addr + j * 1024), "v"(off), "s"(tile) : "memory", "m0");
+  }
+}
+
+// x as three 16-bit pieces (hi, mid, lo; fp16 or bf16) in the first three contraction slots of an operand slice
+template <bool BF16>
+__device__ __forceinline__ uintx4 three_pieces(float x, bool holder) {
+  unsigned short p[3];
+  float rest = x;
+#pragma unroll
+  for (int i = 0; i < 3; ++i) {
+    if constexpr (BF16) {
+      const __bf16 v = (__bf16)rest;
+      p[i] = __builtin_bit_cast(unsigned short, v);
+      rest -= (float)v;
+    } else {
+      const _Float16 v = (_Float16)rest;
+      p[i] = __builtin_bit_cast(unsigned short, v);
+      rest -= (float)v;
+    }
+  }
+  uintx4 r = {0u, 0u, 0u, 0u};
+  if (holder) { r[0] = (unsigned)p[0] | ((unsigned)p[1] << 16); r[1] = (unsigned)p[2]; }
+  return r;
+}
+
+constexpr int DKDV4_LDS_BYTES = 4 * 64 * 2 * 128 + 4 * 4096;   // two stages of a Q and a dO tile, 4 KB of exchange per wavefront
+template <int D, bool BF16, bool PB>
+__global__ __launch_bounds__(256, 2) void dkdv4_kernel(const BwdParams prm) {
+  static_assert(D == 128, "two 32-column blocks of dK and dV per wavefront");
+  constexpr int KS = D / 16, DBW = D / 64;           // 32-column blocks per wavefront
+  constexpr int TILE_BYTES = 64 * 2 * D, STAGE_BYTES = 2 * TILE_BYTES, EXCH_OFF = 2 * STAGE_BYTES;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+  const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int kh = wv & 1, dh = wv >> 1;
+  const int ln = lane & 31, g = lane >> 5;
+  const int nb = prm.nb;
+  int bh, n;
+  const int per_chunk = gridDim.x / prm.split;
+  const int chunk = blockIdx.x / per_chunk;
+  head_and_block(blockIdx.x - chunk * per_chunk, prm.B * prm.H, nb, bh, n);
+  if (n >= nb) return;
+  const int b = bh / prm.H, h = bh % prm.H;
+  const int mh = (prm.Bm > 1 ? b : 0) * prm.Hm + (prm.Hm > 1 ? h : 0);
+  const cint_ptr_t cp = (cint_ptr_t)(uintptr_t)(prm.col_ptr + (int64_t)mh * nb);
+  const cint_ptr_t rows = (cint_ptr_t)(uintptr_t)prm.row_idx;
+  int u0, u1;
+  {
+    const int t0 = cp[n], len = cp[n + 1] - t0;                // this workgroup's share of the column's list
+    u0 = t0 + (int)((int64_t)len * chunk / prm.split);
+    u1 = t0 + (int)((int64_t)len * (chunk + 1) / prm.split);
+  }
+  const unsigned lds_addr = (unsigned)(uintptr_t)(lds_ptr_t)lds;
+  const unsigned short* qg = (const unsigned short*)prm.q + b * prm.qs[0] + h * prm.qs[1];
+  const unsigned short* gg = (const unsigned short*)prm.d_o + b * prm.dos[0] + h * prm.dos[1];
+  const float* lse_h = prm.lse + (int64_t)bh * prm.N;
+  const float* dlt_h = prm.delta + (int64_t)bh * prm.N;
+  const float inv_scale = 1.0f / prm.sm_scale;
+  // tile copies of step u into `stage`
+  auto issue = [&](int u, int stage) {
+    const int rb = rows[u];
+    const unsigned sa = lds_addr + stage * STAGE_BYTES;
+    part_tile_load_async<4, D, 64>(qg + (int64_t)rb * 64 * prm.qs[2], prm.qs[2], wv, lane, sa);
+    part_tile_load_async<4, D, 64>(gg + (int64_t)rb * 64 * prm.dos[2], prm.dos[2], wv, lane, sa + TILE_BYTES);
+  };
+  // lse and delta of this lane's query (of the wavefront's query block) in step u.  Ordinary loads, asked for
+  // before the step's tile copies and first used after the wait for those copies at the top of the step: the
+  // wait the compiler puts in front of that use then finds nothing in flight.
+  float st_lse = 0.f, st_dlt = 0.f;
+  auto ask_stats = [&](int u) {
+    const int q = rows[u] * 64 + 32 * dh + ln;
+    st_lse = lse_h[q];
+    st_dlt = dlt_h[q];
+  };
+  if (u0 < u1) { ask_stats(u0); issue(u0, 0); }
+
+  const int64_t krow = (int64_t)n * 64 + 32 * kh + ln;
+  const unsigned short* kp = (const unsigned short*)prm.k + b * prm.ks[0] + h * prm.ks[1] + krow * prm.ks[2];
+  const unsigned short* vp = (const unsigned short*)prm.v + b * prm.vs[0] + h * prm.vs[1] + krow * prm.vs[2];
+  uintx4 kfr[KS], vfr[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    kfr[s] = *reinterpret_cast<const uintx4*>(kp + 16 * s + 8 * g);
+    vfr[s] = *reinterpret_cast<const uintx4*>(vp + 16 * s + 8 * g);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // compiler-visible vmcnt(0): K and V are there
+  const float qk_scale = prm.qk_scale;
+  // ones in the three slots the pieces occupy (second operand of the extra slices)
+  const unsigned one16 = BF16 ? 0x3f80u : 0x3c00u;
+  const uintx4 ones_frag = {g == 0 ? (one16 | (one16 << 16)) : 0u, g == 0 ? one16 : 0u, 0u, 0u};
+
+  floatx16 dkacc[DBW], dvacc[DBW];
+#pragma unroll
+  for (int db = 0; db < DBW; ++db) { dkacc[db] = zero16(); dvacc[db] = zero16(); }
+  uintx4* exch_mine = reinterpret_cast<uintx4*>(lds + EXCH_OFF + wv * 4096);
+  const uintx4* exch_partner = reinterpret_cast<const uintx4*>(lds + EXCH_OFF + (wv ^ 2) * 4096);
+  // one block of second products, the 32 queries of block qb against this wavefront's columns, in two parts: the
+  // transposed fragments of dO and Q are read from LDS well ahead of the MFMAs that consume them
+  auto read_cols = [&](const unsigned char* qt, const unsigned char* gt, int qb, uintx4 (&fgt)[2][DBW], uintx4 (&fqt)[2][DBW]) {
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+      for (int db = 0; db < DBW; ++db) {
+        fgt[t2][db] = frag_cols<D, BF16 && !PB>(gt, DBW * dh + db, 2 * qb + t2, lane);
+        fqt[t2][db] = frag_cols<D, BF16 && !PB>(qt, DBW * dh + db, 2 * qb + t2, lane);
+      }
+  };
+  auto second = [&](const uintx4 (&fgt)[2][DBW], const uintx4 (&fqt)[2][DBW], const uintx4 (&pf)[2], const uintx4 (&dsf)[2]) {
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+      for (int db = 0; db < DBW; ++db) {
+        dvacc[db] = mfma_qk<PB>(fgt[t2][db], pf[t2], dvacc[db]);    // dV^T += dO^T P
+        dkacc[db] = mfma_qk<PB>(fqt[t2][db], dsf[t2], dkacc[db]);   // dK^T += Q^T dS
+      }
+  };
+
+  for (int u = u0; u < u1; ++u) {
+    const int stage = (u - u0) & 1;
+    wait_vm<0>();
+    __syncthreads();                 // the step's tiles are complete; everybody has left the previous step
+    // the extra slices of this step from the statistics asked for a step ago; then the next step's
+    const uintx4 lse_slice = three_pieces<BF16>(-st_lse * inv_scale, g == 0);
+    const uintx4 dlt_slice = three_pieces<BF16>(-st_dlt, g == 0);
+    __builtin_amdgcn_sched_barrier(0);
+    if (u + 1 < u1) { ask_stats(u + 1); issue(u + 1, stage ^ 1); }
+    const unsigned char* qt = lds + stage * STAGE_BYTES;
+    const unsigned char* gt = qt + TILE_BYTES;
+
+    // ---- first products of this wavefront's query block: S' = Q K^T - lse / sm_scale, dP' = dO V^T - delta ----
+    floatx16 sacc = zero16(), dpacc = zero16();
+    {
+      // (the fragments in two portions: all sixteen at once do not fit beside K, V and the accumulators)
+#pragma unroll
+      for (int pt = 0; pt < 2; ++pt) {
+        uintx4 fq[KS / 2], fg[KS / 2];
+#pragma unroll
+        for (int s = 0; s < KS / 2; ++s) {
+          fq[s] = frag_rows<D>(qt, 32 * dh, pt * (KS / 2) + s, ln, g);
+          fg[s] = frag_rows<D>(gt, 32 * dh, pt * (KS / 2) + s, ln, g);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < KS / 2; ++s) {
+          sacc = mfma_qk<BF16>(fq[s], kfr[pt * (KS / 2) + s], sacc);
+          dpacc = mfma_qk<BF16>(fg[s], vfr[pt * (KS / 2) + s], dpacc);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      sacc = mfma_qk<BF16>(lse_slice, ones_frag, sacc);
+      dpacc = mfma_qk<BF16>(dlt_slice, ones_frag, dpacc);
+    }
+    // (the fragments of the own block's second products are on their way while the vector ALU works)
+    uintx4 fgt_own[2][DBW], fqt_own[2][DBW];
+    read_cols(qt, gt, dh, fgt_own, fqt_own);
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- P and dS (rows of the results are queries: register i <-> query 32dh + 8(i/4) + 4g + i%4), packed as
+    // the operand slices of the second products, and handed to the partner ----
+    uintx4 pm[2], dm[2];             // [16-query slice of this wavefront's query block]
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) {
+#pragma unroll
+      for (int jh = 0; jh < 2; ++jh) {
+        const int i0 = 8 * t2 + 4 * jh;
+        float p[4], ds[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          p[e] = __builtin_amdgcn_exp2f(sacc[i0 + e] * qk_scale);
+          ds[e] = p[e] * dpacc[i0 + e];
+        }
+        pm[t2][2 * jh] = pack2<PB>(p[0], p[1]);   pm[t2][2 * jh + 1] = pack2<PB>(p[2], p[3]);
+        dm[t2][2 * jh] = pack2<PB>(ds[0], ds[1]); dm[t2][2 * jh + 1] = pack2<PB>(ds[2], ds[3]);
+      }
+    }
+    // ---- exchange, the second products of the own query block in between ----
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) { exch_mine[(2 * t2) * 64 + lane] = pm[t2]; exch_mine[(2 * t2 + 1) * 64 + lane] = dm[t2]; }
+    uintx4 fgt_oth[2][DBW], fqt_oth[2][DBW];
+    read_cols(qt, gt, 1 - dh, fgt_oth, fqt_oth);
+    __builtin_amdgcn_sched_barrier(0);
+    second(fgt_own, fqt_own, pm, dm);
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    uintx4 pp[2], dp[2];
+#pragma unroll
+    for (int t2 = 0; t2 < 2; ++t2) { pp[t2] = exch_partner[(2 * t2) * 64 + lane]; dp[t2] = exch_partner[(2 * t2 + 1) * 64 + lane]; }
+    second(fgt_oth, fqt_oth, pp, dp);
+  }
+
+  if (prm.split > 1) {   // unscaled fp32 parts; sum_parts_kernel adds them up
+    const int64_t poff = ((int64_t)chunk * prm.B * prm.H + bh) * prm.N * D;
+#pragma unroll
+    for (int db = 0; db < DBW; ++db)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const int64_t off = krow * D + 32 * (DBW * dh + db) + 8 * i4 + 4 * g;
+        store_out4<BF16>(prm.part_dk + poff, off, true, dkacc[db][4 * i4], dkacc[db][4 * i4 + 1], dkacc[db][4 * i4 + 2],
+                         dkacc[db][4 * i4 + 3]);
+        store_out4<BF16>(prm.part_dv + poff, off, true, dvacc[db][4 * i4], dvacc[db][4 * i4 + 1], dvacc[db][4 * i4 + 2],
+                         dvacc[db][4 * i4 + 3]);
+      }
+    return;
+  }
+  const int64_t koffh = b * prm.dks[0] + h * prm.dks[1], voffh = b * prm.dvs[0] + h * prm.dvs[1];
+  void* kbase = prm.out_f32 ? (void*)((float*)prm.dk + koffh) : (void*)((unsigned short*)prm.dk + koffh);
+  void* vbase = prm.out_f32 ? (void*)((float*)prm.dv + voffh) : (void*)((unsigned short*)prm.dv + voffh);
+#pragma unroll
+  for (int db = 0; db < DBW; ++db)
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4) {
+      const int col = 32 * (DBW * dh + db) + 8 * i4 + 4 * g;
+      store_out4<BF16>(kbase, krow * prm.dks[2] + col, prm.out_f32, dkacc[db][4 * i4] * prm.sm_scale, dkacc[db][4 * i4 + 1] * prm.sm_scale,
+                       dkacc[db][4 * i4 + 2] * prm.sm_scale, dkacc[db][4 * i4 + 3] * prm.sm_scale);
+      store_out4<BF16>(vbase, krow * prm.dvs[2] + col, prm.out_f32, dvacc[db][4 * i4], dvacc[db][4 * i4 + 1], dvacc[db][4 * i4 + 2],
+                       dvacc[db][4 * i4 + 3]);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // split > 1: out = scale * sum of the fp32 parts, rounded to the result type.  blockIdx.y: 0 dQ, 1 dK, 2 dV.
 // ---------------------------------------------------------------------------------------
 template <bool BF16>
@@ -667,6 +912,9 @@ static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
                                 hipFuncAttributeMaxDynamicSharedMemorySize, CK::LDS_BYTES);
       (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv_kernel<D, BF16, EW, PB, QB, 1>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, CK::LDS_BYTES);
+    } else if constexpr (D == 128 && !EW) {
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv4_kernel<D, BF16, PB>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, DKDV4_LDS_BYTES);
     } else {
       (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv_kernel<D, BF16, EW, PB, QB, -1>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, CK::LDS_BYTES);
@@ -680,6 +928,8 @@ static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
   if constexpr (D == 256) {   // the two halves of the head dimension of dK, dV in two launches
     hipLaunchKernelGGL((dkdv_kernel<D, BF16, EW, PB, QB, 0>), dim3(grid), dim3(128), CK::LDS_BYTES, st, prm);
     hipLaunchKernelGGL((dkdv_kernel<D, BF16, EW, PB, QB, 1>), dim3(grid), dim3(128), CK::LDS_BYTES, st, prm);
+  } else if constexpr (D == 128 && !EW) {   // block masks at D = 128: four wavefronts per column block, two per SIMD
+    hipLaunchKernelGGL((dkdv4_kernel<D, BF16, PB>), dim3(grid), dim3(256), DKDV4_LDS_BYTES, st, prm);
   } else {
     hipLaunchKernelGGL((dkdv_kernel<D, BF16, EW, PB, QB, -1>), dim3(grid), dim3(128), CK::LDS_BYTES, st, prm);
   }
