@@ -159,6 +159,13 @@ __device__ __forceinline__ floatx16 zero16() {
 }
 
 
+// Values that live in registers through a walking loop (fragments of the stationary operand, row statistics) are
+// passed through here once they have been asked for: the compiler waits for their loads at this point.  Left to
+// itself it moves the loads next to the loop and plants its waits at their first uses inside it, where, being
+// counted waits, they also wait for the tile copies of the next step that have just been issued, in every step.
+__device__ __forceinline__ void settle(uintx4& x) { asm volatile("" : "+v"(x)); }
+__device__ __forceinline__ void settle(float& x) { asm volatile("" : "+v"(x)); }
+
 // Workgroup -> (head, block) for the walking kernels.  Workgroups go to the 8 XCDs round-robin by
 // linear id, and each XCD has its own L2: heads are taken in groups of 8, head i of a group on
 // XCD i, so that the tiles a head's workgroups walk over (K and V, or Q and dO, of that head) are
@@ -230,10 +237,11 @@ __global__ __launch_bounds__(128, D == 256 ? 1 : 2) void dq_kernel(const BwdPara
   }
   // a query without any unmasked key has lse = -inf: every P of its row must come out as 0
   const float lse_q = prm.lse[(int64_t)bh * prm.N + qrow];
-  const float lse2 = EW && lse_q == -INFINITY ? INFINITY : lse_q * kLog2e;
-  const float dlt = prm.delta[(int64_t)bh * prm.N + qrow];
-  // compiler-visible vmcnt(0): everything above has arrived, no vector-memory waits in the loop
-  __builtin_amdgcn_s_waitcnt(0x0F70);
+  float lse2 = EW && lse_q == -INFINITY ? INFINITY : lse_q * kLog2e;
+  float dlt = prm.delta[(int64_t)bh * prm.N + qrow];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) { settle(qfr[s]); settle(dofr[s]); }
+  settle(lse2); settle(dlt);       // everything above has arrived: no vector-memory waits in the loop
   const float qk_scale = prm.qk_scale;
 
   floatx16 dqacc[DB];
@@ -390,7 +398,8 @@ __global__ __launch_bounds__(128, (QB == 1 && D == 64) ? 2 : 1) void dkdv_kernel
     kfr[s] = *reinterpret_cast<const uintx4*>(kp + 16 * s + 8 * g);
     vfr[s] = *reinterpret_cast<const uintx4*>(vp + 16 * s + 8 * g);
   }
-  __builtin_amdgcn_s_waitcnt(0x0F70);   // compiler-visible vmcnt(0), as in dq_kernel
+#pragma unroll
+  for (int s = 0; s < KS; ++s) { settle(kfr[s]); settle(vfr[s]); }   // no vector-memory waits in the loop, as in dq_kernel
   const float qk_scale = prm.qk_scale;
 
   floatx16 dkacc[DB], dvacc[DB];
@@ -717,7 +726,8 @@ __global__ __launch_bounds__(256, 2) void dkdv4_kernel(const BwdParams prm) {
     kfr[s] = *reinterpret_cast<const uintx4*>(kp + 16 * s + 8 * g);
     vfr[s] = *reinterpret_cast<const uintx4*>(vp + 16 * s + 8 * g);
   }
-  __builtin_amdgcn_s_waitcnt(0x0F70);   // compiler-visible vmcnt(0): K and V are there
+#pragma unroll
+  for (int s = 0; s < KS; ++s) { settle(kfr[s]); settle(vfr[s]); }   // K and V are there: no waits for them in the loop
   const float qk_scale = prm.qk_scale;
   // ones in the three slots the pieces occupy (second operand of the extra slices)
   const unsigned one16 = BF16 ? 0x3f80u : 0x3c00u;
