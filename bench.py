@@ -75,7 +75,7 @@ def fwd_bwd_c5(torch, dev, fm, steps, warmup, check=True):
     ff, fb = tiles * 4.0 * TILE * TILE * Dc, tiles * 10.0 * TILE * TILE * Dc
     out = {"workload": "BASELINE configs[4]: fwd+bwd B=2 H=16 N=8192 D=128 bf16, block-causal keep 0.25 shared mask",
            "kept_tiles": tiles,
-           "note": "one bsattn_fwd call and one bsattn_bwd call (delta, dq and dkdv kernels), buffers allocated beforehand"}
+           "note": "one bsattn_fwd call and one bsattn_bwd call (dq kernel, which also computes delta, and dkdv kernel), buffers allocated beforehand"}
     ref = None
     if check:
         from oracle import bsattn_oracle as orc

@@ -4,10 +4,11 @@
 // evaluated over exactly the kept tiles:
 //   delta = rowsum(O * dO);  P = exp(S*sm_scale - lse);  dV = P^T dO;  dP = dO V^T;
 //   dS = P * (dP - delta);   dK = sm_scale * dS^T Q;     dQ = sm_scale * dS K.
-// Three kernels, no atomics, results independent of scheduling:
-//   delta_kernel  one pass over O and dO (HBM bound);
+// Two kernels, no atomics, results independent of scheduling:
 //   dq_kernel     one workgroup (2 wavefronts x 32 queries) per row block, walking the row
 //                 lists: per kept tile  S^T = K Q^T,  dP^T = V dO^T,  dQ^T += K^T dS^T;
+//                 it also computes delta of its queries on the way in (dO is in its registers
+//                 anyway) and leaves it in the workspace for the next kernel;
 //   dkdv_kernel   one workgroup (2 wavefronts x 32 keys) per column block, walking the column
 //                 lists: per kept tile  S = Q K^T,  dP = dO V^T,  dV^T += dO^T P,  dK^T += Q^T dS.
 // Operand roles are chosen so that the fragment a wavefront owns for the whole walk (Q, dO or
@@ -39,37 +40,23 @@ struct BwdParams {
 
 constexpr float kLog2e = 1.4426950408889634f;
 
-// ---------------------------------------------------------------------------------------
-// delta[b,h,n] = sum_d O[n,d] * dO[n,d]   (fa2_bwd.py:17).  8 (D=64) or 16 (D=128) lanes per row.
-// ---------------------------------------------------------------------------------------
-template <int D, bool BF16>
-__global__ __launch_bounds__(256) void delta_kernel(const BwdParams prm) {
-  constexpr int LPR = D / 8;            // lanes per row, 16 bytes each
-  constexpr int RPB = 256 / LPR;        // rows per workgroup
-  const int bh = blockIdx.y, b = bh / prm.H, h = bh % prm.H;
-  const int row = blockIdx.x * RPB + threadIdx.x / LPR, part = threadIdx.x % LPR;
-  if (row >= prm.N) return;
-  const unsigned short* op = (const unsigned short*)prm.o + b * prm.os[0] + h * prm.os[1] + (int64_t)row * prm.os[2] + part * 8;
-  const unsigned short* gp = (const unsigned short*)prm.d_o + b * prm.dos[0] + h * prm.dos[1] + (int64_t)row * prm.dos[2] + part * 8;
-  const uintx4 ov = *reinterpret_cast<const uintx4*>(op);
-  const uintx4 gv = *reinterpret_cast<const uintx4*>(gp);
-  float acc = 0.f;
+// sum of the products of the eight 16-bit elements of a and b
+template <bool BF16>
+__device__ __forceinline__ float dot8(const uintx4& a, const uintx4& b, float acc) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    float o0, o1, g0, g1;
-    const unsigned int ou = ov[i], gu = gv[i];   // by value: bit_cast of a vector element lvalue miscompiles
+    float a0, a1, b0, b1;
+    const unsigned int au = a[i], bu = b[i];   // by value: bit_cast of a vector element lvalue miscompiles
     if constexpr (BF16) {
-      o0 = __builtin_bit_cast(float, ou << 16); o1 = __builtin_bit_cast(float, ou & 0xffff0000u);
-      g0 = __builtin_bit_cast(float, gu << 16); g1 = __builtin_bit_cast(float, gu & 0xffff0000u);
+      a0 = __builtin_bit_cast(float, au << 16); a1 = __builtin_bit_cast(float, au & 0xffff0000u);
+      b0 = __builtin_bit_cast(float, bu << 16); b1 = __builtin_bit_cast(float, bu & 0xffff0000u);
     } else {
-      const half2v oh = __builtin_bit_cast(half2v, ou), gh = __builtin_bit_cast(half2v, gu);
-      o0 = (float)oh[0]; o1 = (float)oh[1]; g0 = (float)gh[0]; g1 = (float)gh[1];
+      const half2v ah = __builtin_bit_cast(half2v, au), bhh = __builtin_bit_cast(half2v, bu);
+      a0 = (float)ah[0]; a1 = (float)ah[1]; b0 = (float)bhh[0]; b1 = (float)bhh[1];
     }
-    acc += o0 * g0 + o1 * g1;
+    acc += a0 * b0 + a1 * b1;
   }
-#pragma unroll
-  for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
-  if (part == 0) prm.delta[(int64_t)bh * prm.N + row] = acc;
+  return acc;
 }
 
 // ---------------------------------------------------------------------------------------
@@ -238,7 +225,17 @@ __global__ __launch_bounds__(128, D == 256 ? 1 : 2) void dq_kernel(const BwdPara
   // a query without any unmasked key has lse = -inf: every P of its row must come out as 0
   const float lse_q = prm.lse[(int64_t)bh * prm.N + qrow];
   float lse2 = EW && lse_q == -INFINITY ? INFINITY : lse_q * kLog2e;
-  float dlt = prm.delta[(int64_t)bh * prm.N + qrow];
+  // delta = rowsum(O * dO) (fa2_bwd.py:17): the lane holds one half of its query's row of dO, its neighbour 32
+  // lanes on the other half.  Also kept for the dK/dV kernel, which needs it by key tile.
+  float dlt;
+  {
+    const unsigned short* op = (const unsigned short*)prm.o + b * prm.os[0] + h * prm.os[1] + qrow * prm.os[2];
+    float acc = 0.f;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) acc = dot8<BF16>(*reinterpret_cast<const uintx4*>(op + 16 * s + 8 * g), dofr[s], acc);
+    dlt = acc + __shfl_xor(acc, 32);
+    if (chunk == 0 && g == 0) prm.delta[(int64_t)bh * prm.N + qrow] = dlt;
+  }
 #pragma unroll
   for (int s = 0; s < KS; ++s) { settle(qfr[s]); settle(dofr[s]); }
   settle(lse2); settle(dlt);       // everything above has arrived: no vector-memory waits in the loop
@@ -931,8 +928,6 @@ static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
     }
   });
   const int BH = prm.B * prm.H;
-  constexpr int RPB = 256 / (D / 8);
-  hipLaunchKernelGGL((delta_kernel<D, BF16>), dim3((prm.N + RPB - 1) / RPB, BH), dim3(256), 0, st, prm);
   const int grid = ((BH + 7) / 8) * 8 * prm.nb * prm.split;   // heads in groups of 8, the last group padded
   hipLaunchKernelGGL((dq_kernel<D, BF16, EW, PB, KB>), dim3(grid), dim3(128), CQ::LDS_BYTES, st, prm);
   if constexpr (D == 256) {   // the two halves of the head dimension of dK, dV in two launches
