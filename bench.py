@@ -55,11 +55,14 @@ def event_times(fn, iters, warmup, torch):
     return sorted(a.elapsed_time(b) for a, b in evs)       # ms
 
 
-def fwd_bwd_c5(torch, dev, fm, steps, warmup, check=True):
+def fwd_bwd_c5(torch, dev, fm, steps, warmup, check=True, uniform=0):
     """HIP-event times of one forward call and one backward call at configs[4], in both output modes:
     results typed bf16 like the inputs (what autograd hands back; P and dS rounded to bf16) and results in
     fp32 (P and dS kept in fp16).  With check: relative L2 errors of O, dQ, dK, dV against the oracle
-    (numpy fp32 closed-form gradients) on two of the 32 heads."""
+    (numpy fp32 closed-form gradients) on two of the 32 heads.
+    uniform = L > 0 replaces the mask of configs[4] by one with exactly L kept tiles in every row and every
+    column (row r keeps the columns r + 7 j mod 128, j < L): the time of a launch as a function of the list
+    length separates what a launch costs per tile from what it costs per workgroup."""
     import numpy as np
     B, H, Nc, Dc = 2, 16, 8192, 128
     nbc = Nc // TILE
@@ -67,13 +70,19 @@ def fwd_bwd_c5(torch, dev, fm, steps, warmup, check=True):
     q, k, v, do = [torch.randn(B, H, Nc, Dc, generator=g).to(torch.bfloat16) for _ in range(4)]
     m = (torch.rand(1, 1, nbc, nbc, generator=g) < 0.25) | torch.eye(nbc, dtype=torch.bool)
     m = torch.tril(m.reshape(nbc, nbc)).reshape(1, 1, nbc, nbc)
+    if uniform:
+        m = torch.zeros(1, 1, nbc, nbc, dtype=torch.bool)
+        r = torch.arange(nbc)
+        for j in range(uniform):
+            m[0, 0, r, (r + 7 * j) % nbc] = True
     qd, kd, vd, dod, md = [x.to(dev) for x in (q, k, v, do, m)]
     lists = fm.block_mask_to_lists(md)
     lists_t = fm.block_mask_to_lists(md, transpose=True)
     tiles = int(lists.counts[1]) * B * H
     sc = 1.0 / Dc ** 0.5
     ff, fb = tiles * 4.0 * TILE * TILE * Dc, tiles * 10.0 * TILE * TILE * Dc
-    out = {"workload": "BASELINE configs[4]: fwd+bwd B=2 H=16 N=8192 D=128 bf16, block-causal keep 0.25 shared mask",
+    out = {"workload": "BASELINE configs[4]: fwd+bwd B=2 H=16 N=8192 D=128 bf16, block-causal keep 0.25 shared mask"
+                       if not uniform else "shape of BASELINE configs[4] with %d kept tiles in every row and column" % uniform,
            "kept_tiles": tiles,
            "note": "one bsattn_fwd call and one bsattn_bwd call (dq kernel, which also computes delta, and dkdv kernel), buffers allocated beforehand"}
     ref = None
@@ -276,6 +285,9 @@ def main():
     ap.add_argument("--fwd-bwd", action="store_true",
                     help="measurement aid: forward and backward at BASELINE configs[4] (B=2 H=16 N=8192 D=128 bf16, "
                          "block-causal mask with keep 0.25 shared by all heads), then exit")
+    ap.add_argument("--lists-per-row", type=int, default=0,
+                    help="with --fwd-bwd: a mask with exactly this many kept tiles in every row and column "
+                         "instead of the block-causal one")
     ap.add_argument("--reorder", action="store_true",
                     help="measurement aid: the head-wise token reorder and its inverse, then exit")
     ap.add_argument("--mfma-ceiling", action="store_true",
@@ -309,7 +321,8 @@ def main():
         print(json.dumps(reorder_case(torch, dev, fm)))
         return
     if args.fwd_bwd:
-        print(json.dumps(fwd_bwd_c5(torch, dev, fm, min(args.steps, 50), min(args.warmup, 5), check=not args.no_cpu)))
+        print(json.dumps(fwd_bwd_c5(torch, dev, fm, min(args.steps, 50), min(args.warmup, 5),
+                                    check=not args.no_cpu and not args.lists_per_row, uniform=args.lists_per_row)))
         return
     g = torch.Generator().manual_seed(SEED)
     q, k, v = [torch.randn(1, 1, N, D, generator=g).to(torch.float16) for _ in range(3)]
