@@ -242,7 +242,8 @@ def reorder_case(torch, dev, fm):
 
 
 def mfma_ceiling(torch, dev, iters=8192, launches=10):
-    """Sustained fp16 MFMA rate (TFLOP/s) for two operand patterns, measured with the probe library
+    """Sustained fp16 MFMA rate (TFLOP/s) for two operand patterns and the shader clock the GPU holds
+    meanwhile (cycle counter against wall clock inside the kernel), measured with the probe library
     (probe/mfma_rate.hip in the package directory, built by build.py beside the attention library)."""
     import ctypes
     path = os.path.join(PKG, "probe", "libbsattn_probe.so")
@@ -266,6 +267,7 @@ def mfma_ceiling(torch, dev, iters=8192, launches=10):
                 raise RuntimeError("probe_mfma_rate failed with %d" % rc)
         ts = event_times(run, launches, 3, torch)
         out[name + "_tflops"] = round(flops.value / (ts[len(ts) // 2] * 1e-3) / 1e12, 1)
+        out[name + "_shader_clock_ghz"] = round(float(sink[511].item()), 3)
     out["unit"] = "TFLOP/s"
     out["what"] = "fp16 32x32x16 MFMA only, 2 wavefronts per SIMD, 4 accumulator chains, median of %d launches" % launches
     return out
