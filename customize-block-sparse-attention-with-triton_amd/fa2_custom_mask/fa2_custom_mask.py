@@ -265,6 +265,19 @@ class BackwardPlan:
         return self.dq, self.dk, self.dv
 
 
+def _forward_only(q, k, v, mask, sm_scale, out_fp32, return_lse):
+    """The forward of _attention without anything kept for a backward."""
+    B, H, N, D = _check_qkv(q, k, v, mask)
+    if mask is None:
+        mask = _dense_mask(q.device, num_tiles(N))
+    lists = mask_to_lists(mask, N)
+    q, k, v = _padded(q, N, D), _padded(k, N, D), _padded(v, N, D)
+    o, lse = _forward(q, k, v, lists, sm_scale, torch.float32 if out_fp32 else q.dtype, True)
+    if o.shape[2:] != (N, D):
+        o, lse = o[:, :, :N, :D], lse[:, :, :N]
+    return (o, lse) if return_lse else o
+
+
 class _attention(torch.autograd.Function):
     """forward(q, k, v, mask, sm_scale) as the reference (fa2_custom_mask.py:43-94); two extra
     trailing arguments select an fp32 output and the LSE as second result."""
@@ -313,7 +326,11 @@ def flash_attention_custom_mask(q, k, v, mask=None, sm_scale=1.3):
     returns o like q.  D is 16, 32, 64, 128 or 256; N need not be a multiple of 64 (the last block of a
     block mask then covers the remaining tokens).  Shapes other than D in {64,128,256}, N % 64 == 0
     cost one zero-padded copy of q, k, v per call.  The kept-tile lists of a mask tensor are cached
-    until the tensor is modified."""
+    until the tensor is modified.  When no gradient can be asked for (gradients disabled, or none of q, k, v
+    requires one) the call does not go through torch.autograd.Function, which costs about as much host time
+    as everything else in a small call."""
+    if not (torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)):
+        return _forward_only(q, k, v, mask, sm_scale, False, False)
     return _attention.apply(q, k, v, mask, sm_scale)
 
 
@@ -321,6 +338,8 @@ def flash_attention_custom_mask_lse(q, k, v, mask, sm_scale, out_fp32=False):
     """Same operator, also returning the natural-log logsumexp [B,H,N] fp32 of the kept scaled
     scores; out_fp32=True returns O in fp32.  (Not in the reference, whose second output M is
     only the running maximum: fa2_fwd.py:194-196.)"""
+    if not (torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)):
+        return _forward_only(q, k, v, mask, sm_scale, out_fp32, True)
     return _attention.apply(q, k, v, mask, sm_scale, out_fp32, True)
 
 
