@@ -188,7 +188,8 @@ def config_line(torch, dev, fm, name, N_, keeps, causal, seed, dense_mask_paths,
 def elementwise_case(torch, dev, fm, q, k, v, sm_scale):
     """Token-level causal mask [1,1,N,N] at the headline shape: every diagonal tile is partly set.
     Forward time with the packed mask words applied, and the time of the elementwise preprocessing
-    (reduce + lists + pack of the 307.5 MB mask)."""
+    (reduce + lists + pack of the 307.5 MB mask), also in the form a call with a backward uses (one pass over
+    the mask for the block mask and the packed words of every tile, then row and column lists)."""
     from fa2_custom_mask import utils
     mask = torch.ones(N, N, dtype=torch.bool, device=dev).tril_().reshape(1, 1, N, N)
     lists = utils.mask_to_lists(mask, N)
@@ -200,6 +201,13 @@ def elementwise_case(torch, dev, fm, q, k, v, sm_scale):
         utils.lists_cache.clear()
         utils.mask_to_lists(mask, N)
     tp = event_times(prep, 10, 2, torch)
+
+    def prep_both():   # what a call with a backward does: one pass over the mask, then both list orientations
+        utils.lists_cache.clear()
+        utils.grid_cache.clear()
+        utils.mask_to_lists(mask, N, both=True)
+        utils.mask_to_lists(mask, N, transpose=True)
+    tpb = event_times(prep_both, 10, 2, torch)
     # parity spot check against torch on the first 128 and last 64 queries
     rows = torch.cat([torch.arange(128), torch.arange(N - 64, N)]).to(dev)
     s = (q[0, 0, rows].float() @ k[0, 0].float().T) * sm_scale
@@ -209,7 +217,8 @@ def elementwise_case(torch, dev, fm, q, k, v, sm_scale):
     mf = tf[len(tf) // 2]
     return {"workload": "token-level causal mask, N=17536 D=64 fp16", "kept_tiles": tiles,
             "fwd_ms": round(mf, 5), "fwd_tflops_on_kept_tiles": round(tile_flops(tiles) / mf / 1e9, 1),
-            "preprocess_ms": round(tp[len(tp) // 2], 5), "max_abs_vs_torch_fp32": err}
+            "preprocess_ms": round(tp[len(tp) // 2], 5),
+            "preprocess_for_backward_ms": round(tpb[len(tpb) // 2], 5), "max_abs_vs_torch_fp32": err}
 
 
 def reorder_case(torch, dev, fm):

@@ -357,9 +357,24 @@ __global__ __launch_bounds__(256) void reduce_pack_kernel(const uint8_t* __restr
   }
 }
 
+// The 64 x 64 bit matrix whose row r is the word of lane r, transposed: six rounds of block swaps between lanes
+// l and l ^ j (j = 32 ... 1), each exchanging the off-diagonal j x j blocks of every 2j x 2j block.
+__device__ __forceinline__ unsigned long long transpose64(unsigned long long word, int lane) {
+  unsigned long long keep = 0x00000000ffffffffull;     // columns c with (c & j) == 0
+#pragma unroll
+  for (int j = 32; j >= 1; j >>= 1) {
+    const unsigned lo = __shfl_xor((unsigned)word, j), hi = __shfl_xor((unsigned)(word >> 32), j);
+    const unsigned long long other = ((unsigned long long)hi << 32) | lo;
+    word = (lane & j) ? (word & (keep << j)) | ((other & (keep << j)) >> j)
+                      : (word & keep) | ((other & keep) << j);
+    keep ^= keep << (j >> 1);        // 0x0000ffff0000ffff, 0x00ff00ff..., ..., 0x5555...
+  }
+  return word;
+}
+
 // Words of the kept tiles from their grid positions to their list positions.  TRANSPOSE: the lists are the column
 // lists (list row = column block a, entries = row blocks), and the words are wanted per key with one bit per
-// query: the 64 x 64 bit matrix is transposed with one ballot per word.  One workgroup of four wavefronts per
+// query: the 64 x 64 bit matrix is transposed between the lanes (transpose64).  One workgroup of four wavefronts per
 // GATHER_SPLIT-th of a list row, a wavefront per entry.
 constexpr int GATHER_SPLIT = 4;
 template <bool TRANSPOSE>
@@ -373,21 +388,29 @@ __global__ __launch_bounds__(256) void gather_tiles_kernel(const uint8_t* __rest
   const int a = blockIdx.x / GATHER_SPLIT, sub = blockIdx.x % GATHER_SPLIT, mh = blockIdx.y;
   const int32_t* rp = row_ptr + (int64_t)mh * nb;
   const int t0 = rp[a], t1 = rp[a + 1];
-  for (int t = t0 + sub * 4 + wave; t < t1; t += 4 * GATHER_SPLIT) {
-    const int other = col_idx[t];
-    const int64_t tile = TRANSPOSE ? ((int64_t)mh * nb + other) * nb + a : ((int64_t)mh * nb + a) * nb + other;
-    unsigned long long word = grid_bits[tile * 64 + lane];
-    if constexpr (TRANSPOSE) {
-      unsigned long long out = 0ull;
-#pragma unroll 8
-      for (int r = 0; r < 64; ++r) {
-        const unsigned long long bal = __ballot((word >> r) & 1ull);
-        if (lane == r) out = bal;
+  // four entries of the wavefront in flight: their words are asked for before the first is written
+  constexpr int STEP = 4 * GATHER_SPLIT, FLY = 4;
+  for (int t = t0 + sub * 4 + wave; t < t1; t += STEP * FLY) {
+    unsigned long long word[FLY];
+    uint8_t part[FLY];
+#pragma unroll
+    for (int f = 0; f < FLY; ++f) {
+      const int tt = t + f * STEP;
+      if (tt < t1) {
+        const int other = col_idx[tt];
+        const int64_t tile = TRANSPOSE ? ((int64_t)mh * nb + other) * nb + a : ((int64_t)mh * nb + a) * nb + other;
+        word[f] = grid_bits[tile * 64 + lane];
+        part[f] = grid_partial[tile];
       }
-      word = out;
     }
-    bits[(int64_t)t * 64 + lane] = word;
-    if (lane == 0) partial[t] = grid_partial[tile];
+#pragma unroll
+    for (int f = 0; f < FLY; ++f) {
+      const int tt = t + f * STEP;
+      if (tt < t1) {
+        bits[(int64_t)tt * 64 + lane] = TRANSPOSE ? transpose64(word[f], lane) : word[f];
+        if (lane == 0) partial[tt] = part[f];
+      }
+    }
   }
 }
 
