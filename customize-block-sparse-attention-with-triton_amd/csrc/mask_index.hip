@@ -201,6 +201,21 @@ int launch_quad_lists(const int32_t* row_ptr, const int32_t* col_idx, int Bm, in
   return launch_status();
 }
 
+// The 64 x 64 bit matrix whose row r is the word of lane r, transposed: six rounds of block swaps between lanes
+// l and l ^ j (j = 32 ... 1), each exchanging the off-diagonal j x j blocks of every 2j x 2j block.
+__device__ __forceinline__ unsigned long long transpose64(unsigned long long word, int lane) {
+  unsigned long long keep = 0x00000000ffffffffull;     // columns c with (c & j) == 0
+#pragma unroll
+  for (int j = 32; j >= 1; j >>= 1) {
+    const unsigned lo = __shfl_xor((unsigned)word, j), hi = __shfl_xor((unsigned)(word >> 32), j);
+    const unsigned long long other = ((unsigned long long)hi << 32) | lo;
+    word = (lane & j) ? (word & (keep << j)) | ((other & (keep << j)) >> j)
+                      : (word & keep) | ((other & keep) << j);
+    keep ^= keep << (j >> 1);        // 0x0000ffff0000ffff, 0x00ff00ff..., ..., 0x5555...
+  }
+  return word;
+}
+
 // ---------------------------------------------------------------------------------------
 // Elementwise masks: the 64 x 64 bools of every kept tile packed into 64 words of 64 bits
 // (word r = row r of the tile, bit c = column c), plus a flag per kept tile saying whether the
@@ -230,7 +245,7 @@ __device__ __forceinline__ unsigned bools16(const u32x4& d) {
 // memory row): one load instruction covers 16 / G memory rows of the G tiles, 16 bytes per lane.  The four
 // lanes that share a memory row of a tile put their bits together, the words go through LDS so that lane l
 // ends up with the word of memory row l of each tile.  In MODE 1 that is bit r of the words to come for
-// column l: the 64 x 64 bit matrix is transposed with one ballot per word.
+// column l: the 64 x 64 bit matrix is transposed between the lanes (transpose64).
 template <int MODE, int G>
 __global__ __launch_bounds__(256) void pack_tiles_kernel(const uint8_t* __restrict__ dense, int nb, int H,
                                                          int64_t sb, int64_t sh, int64_t sm, int64_t sn,
@@ -284,15 +299,7 @@ __global__ __launch_bounds__(256) void pack_tiles_kernel(const uint8_t* __restri
       for (int jj = 0; jj < G; ++jj) {
         if (tg + jj >= t1) break;
         unsigned long long word = my[jj][lane];
-        if constexpr (MODE == 1) {
-          unsigned long long out = 0ull;
-#pragma unroll 8
-          for (int r = 0; r < 64; ++r) {
-            const unsigned long long b = __ballot((word >> r) & 1ull);
-            if (lane == r) out = b;
-          }
-          word = out;
-        }
+        if constexpr (MODE == 1) word = transpose64(word, lane);
         bits[(int64_t)(tg + jj) * 64 + lane] = word;
         const bool full = __ballot(word == ~0ull) == ~0ull;
         if (lane == 0) partial[tg + jj] = full ? 0 : 1;
@@ -355,21 +362,6 @@ __global__ __launch_bounds__(256) void reduce_pack_kernel(const uint8_t* __restr
     if (any) grid_bits[tile * 64 + lane] = word;        // (tiles without a set element are never looked at)
     if (lane == 0) { block[tile] = any ? 1 : 0; grid_partial[tile] = any && !full ? 1 : 0; }
   }
-}
-
-// The 64 x 64 bit matrix whose row r is the word of lane r, transposed: six rounds of block swaps between lanes
-// l and l ^ j (j = 32 ... 1), each exchanging the off-diagonal j x j blocks of every 2j x 2j block.
-__device__ __forceinline__ unsigned long long transpose64(unsigned long long word, int lane) {
-  unsigned long long keep = 0x00000000ffffffffull;     // columns c with (c & j) == 0
-#pragma unroll
-  for (int j = 32; j >= 1; j >>= 1) {
-    const unsigned lo = __shfl_xor((unsigned)word, j), hi = __shfl_xor((unsigned)(word >> 32), j);
-    const unsigned long long other = ((unsigned long long)hi << 32) | lo;
-    word = (lane & j) ? (word & (keep << j)) | ((other & (keep << j)) >> j)
-                      : (word & keep) | ((other & keep) << j);
-    keep ^= keep << (j >> 1);        // 0x0000ffff0000ffff, 0x00ff00ff..., ..., 0x5555...
-  }
-  return word;
 }
 
 // Words of the kept tiles from their grid positions to their list positions.  TRANSPOSE: the lists are the column
