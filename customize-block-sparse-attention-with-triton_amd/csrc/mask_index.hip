@@ -220,12 +220,20 @@ __device__ __forceinline__ unsigned long long transpose64(unsigned long long wor
 // Elementwise masks: the 64 x 64 bools of every kept tile packed into 64 words of 64 bits
 // (word r = row r of the tile, bit c = column c), plus a flag per kept tile saying whether the
 // tile is only partly set.  Slot t of `bits` / `partial` belongs to entry t of the kept-tile
-// list.  PACK_SPLIT workgroups of 4 wavefronts per mask row block, their wavefronts striding over
-// the row block's kept tiles (a wavefront has one tile's loads in flight at a time, so the
-// kernel lives on the number of wavefronts); lane l packs row l of the tile.  With the row and column strides of the mask and the
-// lists both transposed, the words describe the columns (what the dK/dV pass needs).
+// list.  `split` workgroups of 4 wavefronts per mask row block, their wavefronts striding over
+// the row block's kept tiles; lane l packs row l of the tile.  A wavefront has one turn's loads in
+// flight at a time, so the kernel lives on the number of wavefronts: `split` is chosen so that even
+// a full row gives every wavefront a single turn (every tile of a 17536 x 17536 mask kept: 64 us
+// against 72 us with 8 workgroups per row).  With the row and
+// column strides of the mask and the lists both transposed, the words describe the columns (what the
+// dK/dV pass needs).
 // ---------------------------------------------------------------------------------------
-constexpr int PACK_SPLIT = 8;
+constexpr int PACK_SPLIT_MAX = 32;
+// workgroups per mask row block: a full row of nb tiles gives every wavefront one turn of `per_turn` tiles
+static int pack_split(int nb, int per_turn) {
+  const int s = (nb + 4 * per_turn - 1) / (4 * per_turn);
+  return s < 1 ? 1 : s > PACK_SPLIT_MAX ? PACK_SPLIT_MAX : s;
+}
 constexpr int PACK_G = 4;     // measured against 8 and 16: fewer, longer wavefronts lose more than longer runs gain
 
 // 16 bool bytes (each 0 or 1) -> 16 bits: a dot product of four bytes with (1, 2, 4, 8) or (16, 32, 64, 128)
@@ -252,16 +260,22 @@ __global__ __launch_bounds__(256) void pack_tiles_kernel(const uint8_t* __restri
                                                          const int32_t* __restrict__ row_ptr,
                                                          const int32_t* __restrict__ col_idx,
                                                          uint8_t* __restrict__ partial,
-                                                         unsigned long long* __restrict__ bits) {
+                                                         unsigned long long* __restrict__ bits, int split) {
   __shared__ unsigned long long stage[MODE == 2 ? 1 : 4][MODE == 2 ? 1 : G][64];      // [wavefront][tile of the group][memory row]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   // (row blocks from the last to the first: with causal masks the long lists then start first)
-  const int rb = nb - 1 - blockIdx.x / PACK_SPLIT, sub = blockIdx.x % PACK_SPLIT, bh = blockIdx.y;
+  const int rb = nb - 1 - blockIdx.x / split, bh = blockIdx.y;
+  // Workgroups go to the 8 XCDs round-robin.  With a split that is a multiple of 8 an unrotated share index ties
+  // every XCD, and its L2, to the same byte ranges of all memory rows of the mask; rotating the shares by the row
+  // block spreads them (measured at N = 17536, token-causal mask: 28.7 against 32.9 us with 8 shares; without the
+  // rotation 14, 18 and 20 shares were fast and 8 and 16 slow).  The transposing mode measured the other way round
+  // (8, 16, 24 shares unrotated: 41-44 us; 12, 18, 32: 51-56 us) and keeps the tie.
+  const int sub = MODE == 1 ? blockIdx.x % split : (blockIdx.x + rb) % split;
   const int32_t* rp = row_ptr + (int64_t)bh * nb;
   const int t0 = rp[rb], t1 = rp[rb + 1];
   const uint8_t* head = dense + (bh / H) * sb + (bh % H) * sh + (int64_t)rb * 64 * sm;
   if constexpr (MODE == 2) {
-    for (int t = t0 + sub * 4 + wave; t < t1; t += 4 * PACK_SPLIT) {
+    for (int t = t0 + sub * 4 + wave; t < t1; t += 4 * split) {
       const uint8_t* p = head + (int64_t)col_idx[t] * 64 * sn + lane * sm;
       unsigned long long word = 0ull;
       for (int c = 0; c < 64; ++c) word |= (unsigned long long)(p[(int64_t)c * sn] != 0) << c;
@@ -275,7 +289,7 @@ __global__ __launch_bounds__(256) void pack_tiles_kernel(const uint8_t* __restri
     const int64_t step = 64 * sn;                    // offset of a tile = its column block times this
     const int sub_row = lane / (4 * G), j = (lane >> 2) % G, chunk = lane & 3;
     unsigned long long (*my)[64] = stage[wave];
-    for (int tg = t0 + G * (sub * 4 + wave); tg < t1; tg += 4 * G * PACK_SPLIT) {
+    for (int tg = t0 + G * (sub * 4 + wave); tg < t1; tg += 4 * G * split) {
       const int tj = tg + j < t1 ? tg + j : t1 - 1;               // (a group past the end repeats the last tile)
       const uint8_t* p = head + (int64_t)col_idx[tj] * step + (int64_t)sub_row * S + 16 * chunk;
 #pragma unroll 1
@@ -484,13 +498,16 @@ int launch_pack_tiles(const uint8_t* dense, int Bm, int Hm, int nb, int64_t sb, 
                       unsigned long long* bits, hipStream_t st) {
   // the wide loads need 16-byte aligned memory rows
   const bool wide = (((uintptr_t)dense | (uintptr_t)sb | (uintptr_t)sh) & 15) == 0;
-  const dim3 grid(nb * PACK_SPLIT, Bm * Hm);
-  if (wide && sn == 1 && sm % 16 == 0)
-    hipLaunchKernelGGL((pack_tiles_kernel<0, PACK_G>), grid, dim3(256), 0, st, dense, nb, Hm, sb, sh, sm, sn, row_ptr, col_idx, partial, bits);
-  else if (wide && sm == 1 && sn % 16 == 0)
-    hipLaunchKernelGGL((pack_tiles_kernel<1, 4>), grid, dim3(256), 0, st, dense, nb, Hm, sb, sh, sm, sn, row_ptr, col_idx, partial, bits);
-  else
-    hipLaunchKernelGGL((pack_tiles_kernel<2, 1>), grid, dim3(256), 0, st, dense, nb, Hm, sb, sh, sm, sn, row_ptr, col_idx, partial, bits);
+  if (wide && sn == 1 && sm % 16 == 0) {
+    const int split = pack_split(nb, PACK_G);
+    hipLaunchKernelGGL((pack_tiles_kernel<0, PACK_G>), dim3(nb * split, Bm * Hm), dim3(256), 0, st, dense, nb, Hm, sb, sh, sm, sn, row_ptr, col_idx, partial, bits, split);
+  } else if (wide && sm == 1 && sn % 16 == 0) {
+    const int split = 8;      // (see the kernel)
+    hipLaunchKernelGGL((pack_tiles_kernel<1, 4>), dim3(nb * split, Bm * Hm), dim3(256), 0, st, dense, nb, Hm, sb, sh, sm, sn, row_ptr, col_idx, partial, bits, split);
+  } else {
+    const int split = 8;
+    hipLaunchKernelGGL((pack_tiles_kernel<2, 1>), dim3(nb * split, Bm * Hm), dim3(256), 0, st, dense, nb, Hm, sb, sh, sm, sn, row_ptr, col_idx, partial, bits, split);
+  }
   return launch_status();
 }
 
