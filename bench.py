@@ -223,6 +223,10 @@ def elementwise_case(torch, dev, fm, q, k, v, sm_scale):
         utils.mask_to_lists(mask, N, both=True)
         utils.mask_to_lists(mask, N, transpose=True)
     tpb = event_times(prep_both, 10, 2, torch)
+    # pack_tiles_kernel alone: the 64 x 64 bytes of every kept tile in, 512 bytes of words and a flag byte out
+    tk = event_times(lambda: utils.pack_mask_tiles(mask, lists), 20, 3, torch)
+    mk = tk[len(tk) // 2]
+    pack_bytes = tiles * (4096 + 513)
     # parity spot check against torch on the first 128 and last 64 queries
     rows = torch.cat([torch.arange(128), torch.arange(N - 64, N)]).to(dev)
     s = (q[0, 0, rows].float() @ k[0, 0].float().T) * sm_scale
@@ -233,7 +237,11 @@ def elementwise_case(torch, dev, fm, q, k, v, sm_scale):
     return {"workload": "token-level causal mask, N=17536 D=64 fp16", "kept_tiles": tiles,
             "fwd_ms": round(mf, 5), "fwd_tflops_on_kept_tiles": round(tile_flops(tiles) / mf / 1e9, 1),
             "preprocess_ms": round(tp[len(tp) // 2], 5),
-            "preprocess_for_backward_ms": round(tpb[len(tpb) // 2], 5), "max_abs_vs_torch_fp32": err}
+            "preprocess_for_backward_ms": round(tpb[len(tpb) // 2], 5),
+            "pack_tiles": {"ms": round(mk, 5), "bytes": pack_bytes, "GBps": round(pack_bytes / mk / 1e6, 1),
+                           "frac_hbm_peak": round(pack_bytes / mk / 1e6 / PEAK_HBM_GBS, 4),
+                           "what": "bsattn_pack_mask_tiles over all kept tiles by their row lists, host wrapper included"},
+            "max_abs_vs_torch_fp32": err}
 
 
 def reorder_case(torch, dev, fm):
