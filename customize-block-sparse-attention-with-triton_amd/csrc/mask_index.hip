@@ -381,21 +381,23 @@ __global__ __launch_bounds__(256) void reduce_pack_kernel(const uint8_t* __restr
 // Words of the kept tiles from their grid positions to their list positions.  TRANSPOSE: the lists are the column
 // lists (list row = column block a, entries = row blocks), and the words are wanted per key with one bit per
 // query: the 64 x 64 bit matrix is transposed between the lanes (transpose64).  One workgroup of four wavefronts per
-// GATHER_SPLIT-th of a list row, a wavefront per entry.
-constexpr int GATHER_SPLIT = 4;
+// `split`-th of a list row, a wavefront per entry, four entries of a wavefront in flight; as in pack_tiles_kernel
+// the shares are as many as give every wavefront of a full list one turn, and rotated by the list row.
+constexpr int GATHER_FLY = 4;
 template <bool TRANSPOSE>
 __global__ __launch_bounds__(256) void gather_tiles_kernel(const uint8_t* __restrict__ grid_partial,
                                                            const unsigned long long* __restrict__ grid_bits, int nb,
                                                            const int32_t* __restrict__ row_ptr,
                                                            const int32_t* __restrict__ col_idx,
                                                            uint8_t* __restrict__ partial,
-                                                           unsigned long long* __restrict__ bits) {
+                                                           unsigned long long* __restrict__ bits, int split) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int a = blockIdx.x / GATHER_SPLIT, sub = blockIdx.x % GATHER_SPLIT, mh = blockIdx.y;
+  const int a = blockIdx.x / split, sub = (blockIdx.x + a) % split, mh = blockIdx.y;
   const int32_t* rp = row_ptr + (int64_t)mh * nb;
   const int t0 = rp[a], t1 = rp[a + 1];
   // four entries of the wavefront in flight: their words are asked for before the first is written
-  constexpr int STEP = 4 * GATHER_SPLIT, FLY = 4;
+  constexpr int FLY = GATHER_FLY;
+  const int STEP = 4 * split;
   for (int t = t0 + sub * 4 + wave; t < t1; t += STEP * FLY) {
     unsigned long long word[FLY];
     uint8_t part[FLY];
@@ -432,11 +434,12 @@ int launch_reduce_pack(const uint8_t* dense, int Bm, int Hm, int N, int64_t sb, 
 int launch_gather_tiles(const uint8_t* grid_partial, const unsigned long long* grid_bits, int Bm, int Hm, int nb,
                         int transposed, const int32_t* row_ptr, const int32_t* col_idx, uint8_t* partial,
                         unsigned long long* bits, hipStream_t st) {
-  const dim3 grid(nb * GATHER_SPLIT, Bm * Hm);
+  const int split = pack_split(nb, GATHER_FLY);
+  const dim3 grid(nb * split, Bm * Hm);
   if (transposed)
-    hipLaunchKernelGGL(gather_tiles_kernel<true>, grid, dim3(256), 0, st, grid_partial, grid_bits, nb, row_ptr, col_idx, partial, bits);
+    hipLaunchKernelGGL(gather_tiles_kernel<true>, grid, dim3(256), 0, st, grid_partial, grid_bits, nb, row_ptr, col_idx, partial, bits, split);
   else
-    hipLaunchKernelGGL(gather_tiles_kernel<false>, grid, dim3(256), 0, st, grid_partial, grid_bits, nb, row_ptr, col_idx, partial, bits);
+    hipLaunchKernelGGL(gather_tiles_kernel<false>, grid, dim3(256), 0, st, grid_partial, grid_bits, nb, row_ptr, col_idx, partial, bits, split);
   return launch_status();
 }
 
