@@ -5,6 +5,16 @@
 
 namespace bsattn {
 
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// 16 bool bytes (each 0 or 1) -> 16 bits: a dot product of four bytes with (1, 2, 4, 8) or (16, 32, 64, 128)
+// places four bits at once
+__device__ __forceinline__ unsigned bools16(const u32x4& d) {
+  const unsigned lo = __builtin_amdgcn_udot4(d[1], 0x80402010u, __builtin_amdgcn_udot4(d[0], 0x08040201u, 0u, false), false);
+  const unsigned hi = __builtin_amdgcn_udot4(d[3], 0x80402010u, __builtin_amdgcn_udot4(d[2], 0x08040201u, 0u, false), false);
+  return lo | (hi << 8);
+}
+
 // ---------------------------------------------------------------------------------------
 // dense [.,.,N,N] bool -> block [.,.,nb,nb] bool (tile kept iff any element set).
 // One wavefront owns 64 rows x 1024 columns (16 tiles): every lane ORs its 16-byte column
@@ -110,6 +120,109 @@ __global__ __launch_bounds__(256) void fill_rows_kernel(const uint8_t* __restric
     int32_t* g = groups + (int64_t)gidx[row] * 5;
     g[0] = bh / H; g[1] = bh % H; g[2] = m; g[3] = start; g[4] = pos - start;
   }
+}
+
+
+// ---------------------------------------------------------------------------------------
+// Counting and scanning in one workgroup, for contiguous block masks of up to 1023 rows and 256 KB (one launch
+// less: at 274 rows the launches and the gaps between them are nearly all of the 12 us the three steps take).
+// In row-major order the kept tiles of a contiguous mask are a stream compaction of its bytes: thread t owns
+// the `seg` consecutive bytes from t * seg (16-byte loads, held in registers), the block-wide exclusive scan of
+// the threads' counts gives the number of kept tiles in front of a thread's segment, and the segments stay in
+// LDS with one bit per byte: thread r then finds the start of row r as the count in front of the segment that
+// holds byte r * nb plus the set bits of that segment below it.  Lengths and the rows' positions in `groups`
+// follow from the starts after a second scan over the non-empty flags.
+// fill_rows_kernel then writes col_idx and groups with the whole GPU (one workgroup writing 75 000 scattered
+// entries takes 50 us).
+// ---------------------------------------------------------------------------------------
+constexpr int LISTS_ONE_MAX_ROWS = 1023, LISTS_ONE_MAX_SEG = 256;
+
+// inclusive sum over the 1024 threads of the workgroup; s_w: 16 ints of LDS; returns the sum, *total = all
+__device__ __forceinline__ int block_inclusive_sum(int v, int* s_w, int* total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int o = __shfl_up(v, off);
+    if (lane >= off) v += o;
+  }
+  __syncthreads();                      // s_w may still be read from the previous use
+  if (lane == 63) s_w[wave] = v;
+  __syncthreads();
+  int before = 0, all = 0;
+#pragma unroll
+  for (int w = 0; w < 16; ++w) {
+    const int t = s_w[w];
+    if (w < wave) before += t;
+    all += t;
+  }
+  *total = all;
+  return v + before;
+}
+
+__global__ __launch_bounds__(1024) void count_scan_kernel(const uint8_t* __restrict__ block, int rows, int nb,
+                                                          int seg, int32_t* __restrict__ row_ptr,
+                                                          int32_t* __restrict__ gidx, int32_t* __restrict__ counts) {
+  constexpr int CH = LISTS_ONE_MAX_SEG / 16, WORDS = (CH + 1) / 2;
+  __shared__ int s_w[16];
+  __shared__ int s_off[1024];                   // kept tiles in front of a thread's segment
+  __shared__ unsigned s_bits[1024][WORDS];      // a thread's segment, one bit per byte
+  __shared__ int s_start[LISTS_ONE_MAX_ROWS + 1];
+  const int tid = threadIdx.x;
+  const int total = rows * nb, base = tid * seg;
+  unsigned bits[WORDS];
+#pragma unroll
+  for (int w = 0; w < WORDS; ++w) bits[w] = 0u;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int off = base + 16 * c;
+    if (16 * c < seg && off < total) {
+      u32x4 d = {0u, 0u, 0u, 0u};
+      if (off + 16 <= total) {
+        d = *reinterpret_cast<const u32x4*>(block + off);
+      } else {                            // the last, incomplete chunk of the mask: byte by byte
+#pragma unroll
+        for (int b = 0; b < 16; ++b)
+          if (off + b < total) d[b >> 2] |= (unsigned)block[off + b] << (8 * (b & 3));
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {       // every byte -> 0 / 1 (any non-zero byte counts as set)
+        unsigned t = d[i];
+        t |= t >> 4; t |= t >> 2; t |= t >> 1;
+        d[i] = t & 0x01010101u;
+      }
+      bits[c >> 1] |= bools16(d) << (16 * (c & 1));
+    }
+  }
+  int cnt = 0;
+#pragma unroll
+  for (int w = 0; w < WORDS; ++w) { cnt += __popc(bits[w]); s_bits[tid][w] = bits[w]; }
+  int kept;
+  s_off[tid] = block_inclusive_sum(cnt, s_w, &kept) - cnt;
+  __syncthreads();
+  // thread r: start of row r = kept tiles in front of byte r * nb
+  if (tid <= rows) {
+    int start = kept;
+    if (tid < rows) {
+      const int idx = tid * nb, t = idx / seg, k = idx - t * seg;
+      start = s_off[t];
+#pragma unroll
+      for (int w = 0; w < WORDS; ++w) {
+        const int below = k - 32 * w;     // bits of this word in front of the row's first byte
+        const unsigned m = below <= 0 ? 0u : below >= 32 ? ~0u : (1u << below) - 1u;
+        start += __popc(s_bits[t][w] & m);
+      }
+      row_ptr[tid] = start;
+    } else {
+      row_ptr[rows] = kept; counts[1] = kept;
+    }
+    s_start[tid] = start;
+  }
+  __syncthreads();
+  const int len = tid < rows ? s_start[tid + 1] - s_start[tid] : 0;
+  int ngroups;
+  const int gi = block_inclusive_sum(len > 0 ? 1 : 0, s_w, &ngroups) - (len > 0 ? 1 : 0);
+  if (tid < rows) gidx[tid] = gi;
+  if (tid == 0) counts[0] = ngroups;
 }
 
 
@@ -236,14 +349,6 @@ static int pack_split(int nb, int per_turn) {
 }
 constexpr int PACK_G = 4;     // measured against 8 and 16: fewer, longer wavefronts lose more than longer runs gain
 
-// 16 bool bytes (each 0 or 1) -> 16 bits: a dot product of four bytes with (1, 2, 4, 8) or (16, 32, 64, 128)
-// places four bits at once
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ unsigned bools16(const u32x4& d) {
-  const unsigned lo = __builtin_amdgcn_udot4(d[1], 0x80402010u, __builtin_amdgcn_udot4(d[0], 0x08040201u, 0u, false), false);
-  const unsigned hi = __builtin_amdgcn_udot4(d[3], 0x80402010u, __builtin_amdgcn_udot4(d[2], 0x08040201u, 0u, false), false);
-  return lo | (hi << 8);
-}
 
 // MODE 0: columns are contiguous in memory (sn == 1); MODE 1: rows are (sm == 1: the call for the column
 // lists, with the mask's strides swapped); MODE 2: neither (one byte per load, one tile per wavefront).
@@ -456,12 +561,19 @@ int launch_block_mask_to_lists(const uint8_t* block, int Bm, int Hm, int nb, int
                                int64_t sm, int64_t sn, int32_t* row_ptr, int32_t* col_idx,
                                int32_t* groups, int32_t* counts, int32_t* ws, hipStream_t st) {
   const int rows = Bm * Hm * nb;
+  const int64_t total = (int64_t)rows * nb;
+  const bool contiguous = sn == 1 && sm == nb && (Hm == 1 || sh == (int64_t)nb * nb) &&
+                          (Bm == 1 || sb == (int64_t)Hm * nb * nb) && ((uintptr_t)block & 15) == 0;
   int32_t* cnt = ws;
   int32_t* gidx = ws + rows;
   const dim3 grid((rows + 3) / 4);
-  hipLaunchKernelGGL(count_rows_kernel, grid, dim3(256), 0, st, block, rows, nb, Hm, sb, sh, sm, sn,
-                     cnt);
-  hipLaunchKernelGGL(scan_rows_kernel, dim3(1), dim3(1024), 0, st, cnt, rows, row_ptr, gidx, counts);
+  if (contiguous && rows <= LISTS_ONE_MAX_ROWS && total <= 1024 * LISTS_ONE_MAX_SEG) {
+    const int seg = (((int)total + 1023) / 1024 + 15) / 16 * 16;
+    hipLaunchKernelGGL(count_scan_kernel, dim3(1), dim3(1024), 0, st, block, rows, nb, seg, row_ptr, gidx, counts);
+  } else {
+    hipLaunchKernelGGL(count_rows_kernel, grid, dim3(256), 0, st, block, rows, nb, Hm, sb, sh, sm, sn, cnt);
+    hipLaunchKernelGGL(scan_rows_kernel, dim3(1), dim3(1024), 0, st, cnt, rows, row_ptr, gidx, counts);
+  }
   hipLaunchKernelGGL(fill_rows_kernel, grid, dim3(256), 0, st, block, rows, nb, Hm, sb, sh, sm, sn,
                      row_ptr, gidx, col_idx, groups);
   return launch_status();

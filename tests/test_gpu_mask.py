@@ -25,7 +25,12 @@ def _check_lists(mask_cpu, dev):
 @pytest.mark.parametrize("shape,keep", [((1, 1, 16, 16), 0.5), ((1, 2, 3, 3), 0.4), ((2, 3, 37, 37), 0.1),
                                         ((1, 1, 100, 100), 0.1), ((1, 1, 100, 100), 1.0),
                                         ((1, 1, 274, 274), 0.05), ((2, 16, 128, 128), 0.25),
-                                        ((1, 1, 500, 500), 0.1), ((1, 1, 65, 65), 0.9), ((3, 5, 1, 1), 0.5)])
+                                        ((1, 1, 500, 500), 0.1), ((1, 1, 65, 65), 0.9), ((3, 5, 1, 1), 0.5),
+                                        # either side of the limits of the one-workgroup count and scan
+                                        # (1023 rows, 256 KB of block mask)
+                                        ((1, 1, 512, 512), 0.5), ((1, 1, 513, 513), 0.5), ((1, 1023, 1, 1), 0.5),
+                                        ((1, 1024, 1, 1), 0.5), ((1, 31, 33, 33), 0.3), ((1, 32, 32, 32), 0.3),
+                                        ((1, 1, 512, 512), 1.0), ((2, 2, 255, 255), 0.02)])
 def test_groups_random(dev, shape, keep):
     g = torch.Generator().manual_seed(7)
     _check_lists(torch.rand(*shape, generator=g) < keep, dev)
