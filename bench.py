@@ -302,6 +302,22 @@ def mfma_ceiling(torch, dev, iters=8192, launches=10):
         out[name + "_shader_clock_ghz"] = round(float(sink[511].item()), 3)
     out["unit"] = "TFLOP/s"
     out["what"] = "fp16 32x32x16 MFMA only, 2 wavefronts per SIMD, 4 accumulator chains, median of %d launches" % launches
+    # the same with the forward's softmax instructions beside the MFMAs (probe_mfma_softmax_mix)
+    lib.probe_mfma_softmax_mix.argtypes = lib.probe_mfma_rate.argtypes
+    lib.probe_mfma_softmax_mix.restype = ctypes.c_int
+    flops = ctypes.c_double()
+
+    def run_mix():
+        rc = lib.probe_mfma_softmax_mix(ops.data_ptr(), iters, sink.data_ptr(), ctypes.byref(flops), st)
+        if rc != 0:
+            raise RuntimeError("probe_mfma_softmax_mix failed with %d" % rc)
+    ts = event_times(run_mix, launches, 3, torch)
+    out["with_softmax_instructions"] = {
+        "randn_tflops": round(flops.value / (ts[len(ts) // 2] * 1e-3) / 1e12, 1),
+        "randn_shader_clock_ghz": round(float(sink[511].item()), 3),
+        "what": "per 36 MFMAs 64 v_exp_f32, 32 v_cvt_pk_f16_f32, 32 v_dot2c_f32_f16 and 64 v_fma_f32 on registers "
+                "(the D=64 forward's proportion of vector work; no LDS, memory traffic or barriers): the ceiling "
+                "of the forward's instruction mix on this GPU"}
     return out
 
 

@@ -142,6 +142,16 @@ def test_mfma_rate_probe_runs(dev):
     assert torch.all(sink[:511] == 128.0 * 64)
     # the last slot: the shader clock in GHz the first wavefront saw (cycle counter against the 100 MHz wall clock)
     assert 0.2 < float(sink[511]) < 4.0
+    # the same entry with the forward's softmax instructions beside the MFMAs: 9 MFMAs per iteration
+    lib.probe_mfma_softmax_mix.argtypes = lib.probe_mfma_rate.argtypes
+    g = torch.Generator().manual_seed(3)
+    rnd = torch.randn(4096, generator=g).to(torch.float16).to(dev)
+    sink.fill_(float("nan"))
+    assert lib.probe_mfma_softmax_mix(rnd.data_ptr(), 1 << 21, sink.data_ptr(), None, st) == -8
+    assert lib.probe_mfma_softmax_mix(rnd.data_ptr(), 4, sink.data_ptr(), ctypes.byref(flops), st) == 0
+    torch.cuda.synchronize()
+    assert flops.value == cus * 8 * 4 * 9 * 2 * 32 * 32 * 16
+    assert bool(torch.isfinite(sink).all()) and 0.2 < float(sink[511]) < 4.0
 
 
 def test_committed_toy_fixture(dev):
