@@ -612,7 +612,7 @@ __global__ __launch_bounds__(128, (QB == 1 && D == 64) ? 2 : 1) void dkdv_kernel
 }
 
 // ---------------------------------------------------------------------------------------
-// dK, dV at D = 128 with block masks: workgroup = column block n, four wavefronts (one per SIMD).
+// dK, dV at D = 128: workgroup = column block n, four wavefronts (one per SIMD).
 // Wavefront (kh, dh) owns keys 64n + 32kh + ln and the columns 64dh .. 64dh + 63 of their dK and dV rows: half
 // the accumulators of dkdv_kernel's wavefront, which, with K, V, dK and dV of its keys in 192 of 512
 // registers, runs alone on its SIMD and leaves the matrix cores idle two thirds of the time.  Here a wavefront
@@ -665,7 +665,7 @@ __device__ __forceinline__ uintx4 three_pieces(float x, bool holder) {
 }
 
 constexpr int DKDV4_LDS_BYTES = 4 * 64 * 2 * 128 + 4 * 4096;   // two stages of a Q and a dO tile, 4 KB of exchange per wavefront
-template <int D, bool BF16, bool PB>
+template <int D, bool BF16, bool PB, bool EW>
 __global__ __launch_bounds__(256, 2) void dkdv4_kernel(const BwdParams prm) {
   static_assert(D == 128, "two 32-column blocks of dK and dV per wavefront");
   constexpr int KS = D / 16, DBW = D / 64;           // 32-column blocks per wavefront
@@ -706,11 +706,15 @@ __global__ __launch_bounds__(256, 2) void dkdv4_kernel(const BwdParams prm) {
   // lse and delta of this lane's query (of the wavefront's query block) in step u.  Ordinary loads, asked for
   // before the step's tile copies and first used after the wait for those copies at the top of the step: the
   // wait the compiler puts in front of that use then finds nothing in flight.
+  // Elementwise masks: entry u of the column lists has 64 words, one per key of the tile, bit = query; a lane
+  // reads the word of its key the same way.
   float st_lse = 0.f, st_dlt = 0.f;
+  unsigned long long st_bits = 0ull;
   auto ask_stats = [&](int u) {
     const int q = rows[u] * 64 + 32 * dh + ln;
     st_lse = lse_h[q];
     st_dlt = dlt_h[q];
+    if constexpr (EW) st_bits = prm.bits_cols[(int64_t)u * 64 + 32 * kh + ln];
   };
   if (u0 < u1) { ask_stats(u0); issue(u0, 0); }
 
@@ -761,8 +765,12 @@ __global__ __launch_bounds__(256, 2) void dkdv4_kernel(const BwdParams prm) {
     wait_vm<0>();
     __syncthreads();                 // the step's tiles are complete; everybody has left the previous step
     // the extra slices of this step from the statistics asked for a step ago; then the next step's
-    const uintx4 lse_slice = three_pieces<BF16>(-st_lse * inv_scale, g == 0);
+    // (a query without any unmasked key has lse = -inf; all its scores are masked below, whatever the slice holds)
+    const uintx4 lse_slice = three_pieces<BF16>(EW && st_lse == -INFINITY ? 0.f : -st_lse * inv_scale, g == 0);
     const uintx4 dlt_slice = three_pieces<BF16>(-st_dlt, g == 0);
+    // the mask bits of this lane's key for the queries of this wavefront's block, shifted so that bit
+    // 8(i/4) + i%4 belongs to register i
+    const unsigned mw = EW ? (unsigned)(st_bits >> (32 * dh)) >> (4 * g) : 0u;
     __builtin_amdgcn_sched_barrier(0);
     if (u + 1 < u1) { ask_stats(u + 1); issue(u + 1, stage ^ 1); }
     const unsigned char* qt = lds + stage * STAGE_BYTES;
@@ -791,6 +799,7 @@ __global__ __launch_bounds__(256, 2) void dkdv4_kernel(const BwdParams prm) {
       sacc = mfma_qk<BF16>(lse_slice, ones_frag, sacc);
       dpacc = mfma_qk<BF16>(dlt_slice, ones_frag, dpacc);
     }
+    if constexpr (EW) mask_scores(sacc, mw);
     // (the fragments of the own block's second products are on their way while the vector ALU works)
     uintx4 fgt_own[2][DBW], fqt_own[2][DBW];
     read_cols(qt, gt, dh, fgt_own, fqt_own);
@@ -919,8 +928,8 @@ static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
                                 hipFuncAttributeMaxDynamicSharedMemorySize, CK::LDS_BYTES);
       (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv_kernel<D, BF16, EW, PB, QB, 1>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, CK::LDS_BYTES);
-    } else if constexpr (D == 128 && !EW) {
-      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv4_kernel<D, BF16, PB>),
+    } else if constexpr (D == 128) {
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv4_kernel<D, BF16, PB, EW>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, DKDV4_LDS_BYTES);
     } else {
       (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv_kernel<D, BF16, EW, PB, QB, -1>),
@@ -933,8 +942,8 @@ static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
   if constexpr (D == 256) {   // the two halves of the head dimension of dK, dV in two launches
     hipLaunchKernelGGL((dkdv_kernel<D, BF16, EW, PB, QB, 0>), dim3(grid), dim3(128), CK::LDS_BYTES, st, prm);
     hipLaunchKernelGGL((dkdv_kernel<D, BF16, EW, PB, QB, 1>), dim3(grid), dim3(128), CK::LDS_BYTES, st, prm);
-  } else if constexpr (D == 128 && !EW) {   // block masks at D = 128: four wavefronts per column block, two per SIMD
-    hipLaunchKernelGGL((dkdv4_kernel<D, BF16, PB>), dim3(grid), dim3(256), DKDV4_LDS_BYTES, st, prm);
+  } else if constexpr (D == 128) {   // D = 128: four wavefronts per column block, two per SIMD
+    hipLaunchKernelGGL((dkdv4_kernel<D, BF16, PB, EW>), dim3(grid), dim3(256), DKDV4_LDS_BYTES, st, prm);
   } else {
     hipLaunchKernelGGL((dkdv_kernel<D, BF16, EW, PB, QB, -1>), dim3(grid), dim3(128), CK::LDS_BYTES, st, prm);
   }

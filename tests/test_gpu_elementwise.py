@@ -105,7 +105,7 @@ def test_tile_constant_elementwise_equals_block(dev):
                                fm.flash_attention_custom_mask(q, k, v, block.to(dev), 0.125))
 
 
-@pytest.mark.parametrize("D,dtype", [(64, torch.float16), (128, torch.bfloat16)])
+@pytest.mark.parametrize("D,dtype", [(64, torch.float16), (128, torch.bfloat16), (128, torch.float16)])
 def test_backward_elementwise(dev, D, dtype):
     """dQ, dK, dV with elementwise masks (token-causal, and random with empty tiles, full tiles and
     queries without keys) against the oracle's gradient of the naive masked softmax."""
