@@ -914,10 +914,10 @@ static void launch_bwd_t(const BwdParams& prm, hipStream_t st) {
   using C = BwdCfg<D, EW>;
   constexpr int KB = D >= 128 ? 1 : 2;          // dq_kernel walks D >= 128 tiles in two halves (no gain at D = 64: two wavefronts per SIMD anyway)
   using CQ = BwdCfg<D, EW, 32 * KB>;
-  // dkdv_kernel: halves at D = 64 (191 instead of 318 registers: two wavefronts per SIMD; B*H = 32 N = 8192 dense
-  // block-causal backward 1417 -> 1167 us).  At D = 128 it keeps one wavefront per SIMD either way (K, V, dK, dV of
-  // 32 keys are 192 registers) and halves were measured slower (718 against 688 us, C5).
-  constexpr int QB = D == 128 ? 2 : 1;   // (D = 256: halves, and the head dimension of dK, dV in two launches)
+  // dkdv_kernel (D = 64 and 256; D = 128 runs dkdv4_kernel): halves at D = 64 (191 instead of 318 registers: two
+  // wavefronts per SIMD; B*H = 32 N = 8192 dense block-causal backward 1417 -> 1167 us); at D = 256 halves too, and
+  // the head dimension of dK, dV in two launches.
+  constexpr int QB = 1;
   using CK = BwdCfg<D, EW, 32 * QB>;
   static std::atomic<unsigned long long> configured{0};   // raising the dynamic LDS limit is idempotent
   once_per_device(configured, [] {
