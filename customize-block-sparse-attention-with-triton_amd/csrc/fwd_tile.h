@@ -27,6 +27,11 @@ struct FwdParams {
   int out_f32;
   float qk_scale;  // sm_scale * log2(e)
   int64_t qs[3], ks[3], vs[3], os[3];
+  // fwd_kernel: which range of its head workgroup wg takes, for heads with at least perm_min_tiles kept tiles that
+  // are cut into exactly perm_n ranges, the first perm_fast of them with the larger weight (perm_n = 0: none; see
+  // range_permutation)
+  int perm_n, perm_fast, perm_min_tiles;
+  unsigned short perm[512];
 };
 
 // P = exp2(score - m) for the 2 x 16 scores one lane holds of one query (key blocks s0, s1),
