@@ -36,16 +36,17 @@ def test_c3_n17536(dev, keep):
     sampled_forward_check(dev, 17536, 64, uniform_block_mask(1, 1, nb, keep, 1236), 1236, [0, 1, 137, 272, 273])
 
 
-@pytest.mark.parametrize("B,H,N", [(1, 2, 8192), (2, 2, 8192), (1, 4, 4096)])
-def test_dense_few_heads_ranges_dealt_by_phase(dev, B, H, N):
+@pytest.mark.parametrize("B,H,N,D", [(1, 2, 8192, 64), (2, 2, 8192, 64), (1, 4, 4096, 64), (1, 1, 8192, 128), (1, 2, 8192, 128)])
+def test_dense_few_heads_ranges_dealt_by_phase(dev, B, H, N, D):
     """Dense masks with 2 or 4 heads in the launch: every head is cut into ranges that the workgroups take in the
     order of the launcher's range permutation (ranges of like phase on one XCD), as the single dense head of
     test_c3_n17536 is.  Sampled row blocks of every head against the oracle."""
     import fa2_custom_mask as fm
     nb = N // 64
-    q, k, v = make_qkv(B, H, N, 64, torch.float16, 1250 + B * H)
+    q, k, v = make_qkv(B, H, N, D, torch.float16, 1250 + B * H)
     mask = torch.ones(1, 1, nb, nb, dtype=torch.bool)
-    o, lse = fm.flash_attention_custom_mask_lse(q.to(dev), k.to(dev), v.to(dev), mask.to(dev), 0.125)
+    sc = 1.0 / np.sqrt(D)
+    o, lse = fm.flash_attention_custom_mask_lse(q.to(dev), k.to(dev), v.to(dev), mask.to(dev), sc)
     o = o.float().cpu().numpy(); lse = lse.cpu().numpy()
     assert np.isfinite(o).all()
     for b in range(B):
@@ -53,7 +54,7 @@ def test_dense_few_heads_ranges_dealt_by_phase(dev, B, H, N):
             qf, kf, vf = f32(q[b:b + 1, h:h + 1]), f32(k[b:b + 1, h:h + 1]), f32(v[b:b + 1, h:h + 1])
             for mb in (0, nb // 2, nb - 1):
                 r0, r1 = mb * 64, mb * 64 + 64
-                o_ref, lse_ref = c_oracle.naive_fwd(qf, kf, vf, mask.numpy(), 0.125, r0, r1)
+                o_ref, lse_ref = c_oracle.naive_fwd(qf, kf, vf, mask.numpy(), sc, r0, r1)
                 d = o[b, h, r0:r1] - o_ref[0, 0, r0:r1]
                 assert np.abs(d).max() <= 2e-2 and np.linalg.norm(d) / np.linalg.norm(o_ref[0, 0, r0:r1]) <= 1e-3, (b, h, mb)
                 assert np.abs(lse[b, h, r0:r1] - lse_ref[0, 0, r0:r1]).max() <= 2e-3
