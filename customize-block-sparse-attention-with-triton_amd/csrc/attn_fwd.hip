@@ -24,18 +24,16 @@
 // vector ALU out of the way of the matrix cores: the softmax scale is folded into Q, and the
 // running maximum is replaced by a reference exponent that is only moved when needed.
 #include <atomic>
-#include <vector>
-#include <utility>
 #include <mutex>
 #include <map>
 #include <array>
-#include <algorithm>
 #include <chrono>
 #include <cstdlib>
 #include "common.h"
 #include "fwd_split.h"
 #include "fwd_tile.h"
 #include "kernel_util.h"
+#include "range_perm.h"
 
 namespace bsattn {
 
@@ -1009,36 +1007,17 @@ int static_scratch(void** ptr) {
   return BSATTN_OK;
 }
 
-// Range permutation of fwd_kernel.  A head's tile list is cut into W ranges (fwd_split.h: the first F with
-// weight WEIGHT_FAST, the others with WEIGHT_SLOW); range p starts at the fraction split_cum(p) / ctot of the list,
-// which for rows of equal length is the phase frac(split_cum(p) * nb / ctot) of a row.  Workgroups go to the 8 XCDs
-// round-robin by linear id (wg * BH + bh), so workgroup wg of a head sits on the head's XCD number wg % nx,
-// nx = 8 / BH.  Within each weight class (the faster, first-come workgroups keep the larger ranges) the ranges are
-// sorted by phase and dealt out in nx equal runs, one per XCD.  Depends on (nb, W, F, nx) only: kept in a small cache.
+// The range permutation of fwd_kernel (range_perm.h) depends on (nb, W, F, heads) only: kept in a small cache.
 static bool range_permutation(int nb, int W, int F, int BH, unsigned short* out) {
-  if (BH != 1 && BH != 2 && BH != 4) return false;
-  const int nx = 8 / BH;
-  if (W > 512 || W < 2 * nx || F < 0 || F > W || F % nx != 0 || (W - F) % nx != 0) return false;
   static std::mutex mu;
-  static std::map<std::array<int, 4>, std::array<unsigned short, 512>> cache;
-  const std::array<int, 4> key = {nb, W, F, nx};
+  static std::map<std::array<int, 4>, std::array<unsigned short, RANGE_PERM_MAX>> cache;
+  const std::array<int, 4> key = {nb, W, F, BH};
   std::lock_guard<std::mutex> lock(mu);
   auto it = cache.find(key);
   if (it == cache.end()) {
+    std::array<unsigned short, RANGE_PERM_MAX> t{};
+    if (!make_range_permutation(nb, W, F, BH, WEIGHT_FAST, WEIGHT_SLOW, t.data())) return false;
     if (cache.size() >= 64) cache.clear();
-    auto cum = [&](int p) { return p <= F ? (int64_t)WEIGHT_FAST * p : (int64_t)WEIGHT_FAST * F + (int64_t)WEIGHT_SLOW * (p - F); };
-    const int64_t ctot = cum(W);
-    std::array<unsigned short, 512> t{};
-    for (int cls = 0; cls < 2; ++cls) {
-      const int base = cls == 0 ? 0 : F, n = cls == 0 ? F : W - F;
-      if (n == 0) continue;
-      std::vector<std::pair<int64_t, int>> order(n);
-      for (int i = 0; i < n; ++i) order[i] = {(cum(base + i) * nb) % ctot, base + i};
-      std::sort(order.begin(), order.end());
-      for (int i = 0; i < n; ++i) {          // workgroup base + i: XCD (base + i) % nx = i % nx, its i / nx-th of this class
-        t[base + i] = (unsigned short)order[(i % nx) * (n / nx) + i / nx].second;
-      }
-    }
     it = cache.emplace(key, t).first;
   }
   for (int i = 0; i < W; ++i) out[i] = it->second[i];

@@ -31,7 +31,7 @@ struct FwdParams {
   // are cut into exactly perm_n ranges, the first perm_fast of them with the larger weight (perm_n = 0: none; see
   // range_permutation)
   int perm_n, perm_fast, perm_min_tiles;
-  unsigned short perm[512];
+  unsigned short perm[512];        // (RANGE_PERM_MAX of range_perm.h)
 };
 
 // P = exp2(score - m) for the 2 x 16 scores one lane holds of one query (key blocks s0, s1),
