@@ -108,8 +108,14 @@ void fwd_kernel(const FwdParams prm) {
   // all phases of a row, and workgroups that share an XCD, hence an L2, get ranges of like phase, so that they
   // walk the same column blocks at the same time (dense N = 17536, one head: 42 instead of 196 MB fetched from
   // HBM per launch, 104.5 instead of 106.6 us).  The phases are those of rows of equal length: heads that keep less
-  // than three quarters of their tiles are left alone (keep 0.5 measured 2 % slower with the permutation).
-  if (prm.perm_n > 0 && prm.perm_n == hs.Peff && prm.perm_fast == hs.fast && hs.T >= prm.perm_min_tiles) wg = prm.perm[wg];
+  // than three quarters of their tiles are left alone (keep 0.5 measured 2 % slower with the permutation), except
+  // the dense block-causal mask, which has a table of its own (N = 32000: 185 instead of 193 us).
+  if (prm.perm_n > 0 && prm.perm_n == hs.Peff && prm.perm_fast == hs.fast) {
+    if (hs.T >= prm.perm_min_tiles) wg = prm.perm[wg];
+    // the dense block-causal mask (by its number of kept tiles and the length of one row in the middle; a mask
+    // taken for it by mistake merely gets its ranges in another order): ranges sorted by their first column block
+    else if ((int64_t)hs.T * 2 == (int64_t)nb * (nb + 1) && rp[nb / 2 + 1] - rp[nb / 2] == nb / 2 + 1) wg = prm.perm_causal[wg];
+  }
   // Row blocks without kept tiles belong to no range: they are dealt round-robin over all workgroups
   // of the head, which write O = 0, lse = -inf for their share.  (With whole row blocks per
   // wavefront the ranges are row-aligned and cover them, unless the head keeps nothing at all.)
@@ -1008,19 +1014,20 @@ int static_scratch(void** ptr) {
 }
 
 // The range permutation of fwd_kernel (range_perm.h) depends on (nb, W, F, heads) only: kept in a small cache.
-static bool range_permutation(int nb, int W, int F, int BH, unsigned short* out) {
+static bool range_permutation(int nb, int W, int F, int BH, unsigned short* out, unsigned short* out_causal) {
   static std::mutex mu;
-  static std::map<std::array<int, 4>, std::array<unsigned short, RANGE_PERM_MAX>> cache;
+  static std::map<std::array<int, 4>, std::array<unsigned short, 2 * RANGE_PERM_MAX>> cache;
   const std::array<int, 4> key = {nb, W, F, BH};
   std::lock_guard<std::mutex> lock(mu);
   auto it = cache.find(key);
   if (it == cache.end()) {
-    std::array<unsigned short, RANGE_PERM_MAX> t{};
-    if (!make_range_permutation(nb, W, F, BH, WEIGHT_FAST, WEIGHT_SLOW, t.data())) return false;
+    std::array<unsigned short, 2 * RANGE_PERM_MAX> t{};
+    if (!make_range_permutation(nb, W, F, BH, WEIGHT_FAST, WEIGHT_SLOW, false, t.data()) ||
+        !make_range_permutation(nb, W, F, BH, WEIGHT_FAST, WEIGHT_SLOW, true, t.data() + RANGE_PERM_MAX)) return false;
     if (cache.size() >= 64) cache.clear();
     it = cache.emplace(key, t).first;
   }
-  for (int i = 0; i < W; ++i) out[i] = it->second[i];
+  for (int i = 0; i < W; ++i) { out[i] = it->second[i]; out_causal[i] = it->second[RANGE_PERM_MAX + i]; }
   return true;
 }
 
@@ -1041,7 +1048,7 @@ int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
   {
     const int BHl = s.B * s.H;
     const int F = prm.first_ids > 0 && prm.first_ids % BHl == 0 ? (prm.first_ids / BHl < prm.W ? prm.first_ids / BHl : prm.W) : 0;
-    const bool ok = (prm.first_ids == 0 || prm.first_ids % BHl == 0) && range_permutation(prm.nb, prm.W, F, BHl, prm.perm);
+    const bool ok = (prm.first_ids == 0 || prm.first_ids % BHl == 0) && range_permutation(prm.nb, prm.W, F, BHl, prm.perm, prm.perm_causal);
     prm.perm_n = ok ? prm.W : 0;
     prm.perm_fast = F;
     prm.perm_min_tiles = (int)((int64_t)prm.nb * prm.nb * 3 / 4);

@@ -32,6 +32,7 @@ struct FwdParams {
   // range_permutation)
   int perm_n, perm_fast, perm_min_tiles;
   unsigned short perm[512];        // (RANGE_PERM_MAX of range_perm.h)
+  unsigned short perm_causal[512]; // the same for heads whose mask is the dense block-causal one
 };
 
 // P = exp2(score - m) for the 2 x 16 scores one lane holds of one query (key blocks s0, s1),
