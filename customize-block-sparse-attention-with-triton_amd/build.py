@@ -1,5 +1,4 @@
-"""Builds libbsattn.so (gfx950 HIP kernels + C ABI) in-tree with hipcc, and beside it libbsattn_probe.so,
-the benchmark's measurement aid (probe/mfma_rate.hip), which is deliberately not part of the library.
+"""Builds libbsattn.so (gfx950 HIP kernels + C ABI) in-tree with hipcc.
 
 Usage: python build.py [--force]
 """
@@ -11,8 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 LIB = os.path.join(HERE, "fa2_custom_mask", "libbsattn.so")
-PROBE_LIB = os.path.join(HERE, "probe", "libbsattn_probe.so")
-SOURCES = ["api.hip", "mask_index.hip", "attn_fwd.hip", "attn_fwd_pair.hip", "attn_fwd_quad.hip", "attn_bwd.hip", "reorder.hip"]
+SOURCES = ["api.hip", "mask_index.hip", "attn_fwd.hip", "attn_fwd_pair.hip", "attn_bwd.hip", "reorder.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-I" + INCLUDE, "-I" + CSRC,
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",   # no packed fp32 VALU ops
          "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option"]
@@ -43,14 +41,6 @@ def build(force=True, verbose=False):
             print(err)
     cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
     subprocess.check_call(cmd)
-    probe_src = os.path.join(HERE, "probe", "mfma_rate.hip")
-    if force or not os.path.exists(PROBE_LIB) or os.path.getmtime(PROBE_LIB) < os.path.getmtime(probe_src):
-        cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
-               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-               "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option", probe_src, "-o", PROBE_LIB]
-        p = subprocess.run(cmd, stderr=subprocess.PIPE, text=True)
-        if p.returncode != 0:
-            raise RuntimeError("hipcc failed on %s:\n%s" % (probe_src, p.stderr))
     return LIB
 
 

@@ -58,15 +58,6 @@ int bsattn_block_mask_to_lists(const uint8_t* block, int Bm, int Hm, int nb, int
                                     (int32_t*)workspace, (hipStream_t)stream);
 }
 
-int bsattn_quad_lists(const int32_t* row_ptr, const int32_t* col_idx, int Bm, int Hm, int nb, int32_t* quad_ptr,
-                      int32_t* quad_list, int32_t* quad_stats, void* stream) {
-  if (row_ptr == nullptr || col_idx == nullptr || quad_ptr == nullptr || quad_list == nullptr || quad_stats == nullptr)
-    return BSATTN_ERR_NULL;
-  if (Bm <= 0 || Hm <= 0 || nb <= 0) return BSATTN_ERR_SHAPE;
-  if (nb > BSATTN_QUAD_MAX_BLOCKS || (int64_t)Bm * Hm * ((nb + 3) / 4) * nb > 0x7fffffffLL) return BSATTN_ERR_RANGE;
-  return launch_quad_lists(row_ptr, col_idx, Bm, Hm, nb, quad_ptr, quad_list, quad_stats, (hipStream_t)stream);
-}
-
 int bsattn_pack_mask_tiles(const uint8_t* dense, int Bm, int Hm, int N, int64_t sb, int64_t sh, int64_t sm,
                            int64_t sn, const int32_t* row_ptr, const int32_t* col_idx, uint8_t* tile_partial,
                            uint64_t* tile_bits, void* stream) {
@@ -166,6 +157,7 @@ static int fwd_common(const void* q, const void* k, const void* v, void* o, floa
                            v_strides, o_strides);
   if (rc != BSATTN_OK) return rc;
   if (workspace == nullptr || workspace_bytes < coop_workspace_bytes(B, H, N, D)) return BSATTN_ERR_WORKSPACE;
+  if (((uintptr_t)workspace & 15) != 0) return BSATTN_ERR_STRIDE;
   AttnShape s;
   s.B = B; s.H = H; s.N = N; s.D = D; s.Bm = Bm; s.Hm = Hm; s.dtype = dtype; s.out_dtype = out_dtype;
   s.sm_scale = sm_scale;
@@ -199,25 +191,6 @@ int bsattn_fwd_static(const void* q, const void* k, const void* v, void* o, floa
   s.sm_scale = sm_scale;
   for (int i = 0; i < 3; ++i) { s.qs[i] = q_strides[i]; s.ks[i] = k_strides[i]; s.vs[i] = v_strides[i]; s.os[i] = o_strides[i]; s.dos[i] = 0; }
   return launch_fwd(q, k, v, o, lse, row_ptr, col_idx, nullptr, nullptr, s, ws, (hipStream_t)stream);
-}
-
-int bsattn_fwd_quads(const void* q, const void* k, const void* v, void* o, float* lse,
-                     const int32_t* row_ptr, const int32_t* quad_ptr, const int32_t* quad_list, int Bm, int Hm,
-                     int B, int H, int N, int D, int dtype, int out_dtype, float sm_scale,
-                     const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
-                     const int64_t* o_strides, void* workspace, size_t workspace_bytes, void* stream) {
-  if (quad_ptr == nullptr) return BSATTN_ERR_NULL;
-  const int rc = fwd_check(q, k, v, o, row_ptr, quad_list, Bm, Hm, B, H, N, D, dtype, out_dtype, q_strides, k_strides,
-                           v_strides, o_strides);
-  if (rc != BSATTN_OK) return rc;
-  if (D != 64) return BSATTN_ERR_HEAD_DIM;
-  AttnShape s;
-  s.B = B; s.H = H; s.N = N; s.D = D; s.Bm = Bm; s.Hm = Hm; s.dtype = dtype; s.out_dtype = out_dtype;
-  s.sm_scale = sm_scale;
-  for (int i = 0; i < 3; ++i) { s.qs[i] = q_strides[i]; s.ks[i] = k_strides[i]; s.vs[i] = v_strides[i]; s.os[i] = o_strides[i]; s.dos[i] = 0; }
-  if (!quad_supported(s)) return BSATTN_ERR_RANGE;
-  if (workspace == nullptr || workspace_bytes < fwd_workspace_bytes(B, H, N, D)) return BSATTN_ERR_WORKSPACE;
-  return launch_fwd_quads(q, k, v, o, lse, row_ptr, quad_ptr, quad_list, s, workspace, (hipStream_t)stream);
 }
 
 int bsattn_fwd_elementwise(const void* q, const void* k, const void* v, void* o, float* lse,
@@ -271,6 +244,7 @@ static int bwd_common(const void* q, const void* k, const void* v, const void* o
   if ((rc = check_strides(dk_strides, out_bytes, dk)) != BSATTN_OK) return rc;
   if ((rc = check_strides(dv_strides, out_bytes, dv)) != BSATTN_OK) return rc;
   if (workspace == nullptr || workspace_bytes < bwd_workspace_bytes(B, H, N, D)) return BSATTN_ERR_WORKSPACE;
+  if (((uintptr_t)workspace & 15) != 0) return BSATTN_ERR_STRIDE;
   AttnShape s;
   s.B = B; s.H = H; s.N = N; s.D = D; s.Bm = Bm; s.Hm = Hm; s.dtype = dtype; s.out_dtype = out_dtype;
   s.sm_scale = sm_scale;

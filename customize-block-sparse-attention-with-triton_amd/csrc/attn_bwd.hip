@@ -642,11 +642,21 @@ __device__ __forceinline__ void part_tile_load_async(const unsigned short* tile,
   }
 }
 
-// x as three 16-bit pieces (hi, mid, lo; fp16 or bf16) in the first three contraction slots of an operand slice
+// x as three 16-bit pieces (hi, mid, lo; fp16 or bf16) in the first three contraction slots of an operand slice.
+// fp16 pieces hold x / PIECE_GAIN and the other operand of the slice holds PIECE_GAIN instead of ones: lse / sm_scale
+// (about the largest raw q k) and delta = rowsum(O dO) (of the order |dO| sqrt(D), large under loss scaling) may lie
+// far above fp16's 65504, where the first piece would be infinite and the remainders NaN.  With the gain the
+// pieces reach +-4.1e6 (beyond that x is clamped: finite, wrong results instead of NaN) and are exact to
+// max(2^-33 |x|, 2e-6).  bf16 pieces have fp32's range and need no gain.
+constexpr float PIECE_GAIN = 64.0f;
 template <bool BF16>
 __device__ __forceinline__ uintx4 three_pieces(float x, bool holder) {
   unsigned short p[3];
   float rest = x;
+  if constexpr (!BF16) {
+    constexpr float LIM = 65000.0f;
+    rest = fminf(fmaxf(x * (1.0f / PIECE_GAIN), -LIM), LIM);
+  }
 #pragma unroll
   for (int i = 0; i < 3; ++i) {
     if constexpr (BF16) {
@@ -731,7 +741,8 @@ __global__ __launch_bounds__(256, 2) void dkdv4_kernel(const BwdParams prm) {
   for (int s = 0; s < KS; ++s) { settle(kfr[s]); settle(vfr[s]); }   // K and V are there: no waits for them in the loop
   const float qk_scale = prm.qk_scale;
   // ones in the three slots the pieces occupy (second operand of the extra slices)
-  const unsigned one16 = BF16 ? 0x3f80u : 0x3c00u;
+  const unsigned one16 = BF16 ? 0x3f80u : 0x5400u;      // 1.0 (bf16) or PIECE_GAIN = 64.0 (fp16), see three_pieces
+  static_assert(PIECE_GAIN == 64.0f, "0x5400 is 64.0 in fp16");
   const uintx4 ones_frag = {g == 0 ? (one16 | (one16 << 16)) : 0u, g == 0 ? one16 : 0u, 0u, 0u};
 
   floatx16 dkacc[DBW], dvacc[DBW];

@@ -61,17 +61,6 @@ template <int D> struct FwdCfg {
 
 // DT: 0 fp16; 1 bf16 with P rounded to fp16 (V fragments converted); 2 bf16 with P rounded to bf16.
 // CONTIG: the rows of K and of V follow each other without gaps (row stride = D).
-// Measurement build only (-DFWD_TIMELINE, never the library's): wavefront 0 of every workgroup writes the 100 MHz
-// wall clock at a few points to a buffer whose address the launcher takes from the environment variable
-// BSATTN_FWD_TIMELINE: [workgroup][16] = entry, range known, first tile's operands asked for, then per row
-// block segment (up to 4): tiles done, merged in LDS, finished (published or written).
-#ifdef FWD_TIMELINE
-#define FWD_WALL(i) do { if (prm.part_o != nullptr && w == 0 && (i) < 16) \
-    reinterpret_cast<long long*>(prm.part_o)[(int64_t)blockIdx.x * 16 + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
-#else
-#define FWD_WALL(i) do {} while (0)
-#endif
-
 template <int D, int DT, bool ROWS, bool EW, bool CONTIG>
 __global__ __launch_bounds__(FwdCfg<D>::NW * 64, FwdCfg<D>::WG_PER_CU)
 void fwd_kernel(const FwdParams prm) {
@@ -87,7 +76,6 @@ void fwd_kernel(const FwdParams prm) {
 
   const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  FWD_WALL(0);
   const int ln = lane & 31, g = lane >> 5;
   // linear id -> (head, range): heads interleaved, so that every head gets its share of the
   // workgroups that are first on their compute unit
@@ -575,7 +563,6 @@ void fwd_kernel(const FwdParams prm) {
       if (g1 < hs.lo + hs.T) g1 = snap_boundary<C::SNAP>(g1, s1, e1);
       if (g0 >= g1) return;
     }
-    FWD_WALL(1);
     stage_cols(g0, g1);
     if (threadIdx.x == 0) { ctr[0] = g0 + 2 * NW; ctr[3] = 0; }
     __syncthreads();
@@ -584,7 +571,6 @@ void fwd_kernel(const FwdParams prm) {
     int cb_nxt = nxt < g1 ? __builtin_amdgcn_readfirstlane(col_of(nxt)) : 0;   // column block of tile nxt
     int kdone = -1, vdone = -1;
     int t = g0;
-    int nseg = 0;   // (segments done: only read by the measurement build)
     const int32_t* rpg = prm.row_ptr + (int64_t)mh * nb;
     while (t < g1) {
       const int row_s = rp[r], row_e = rp[r + 1];
@@ -629,7 +615,6 @@ void fwd_kernel(const FwdParams prm) {
         if (kdone != cur) { k_copy_all(kg + (int64_t)(cx & COL_MASK) * 64 * k_rs, cur); kdone = cur; }
         if (vdone != cur) { v_copy_all(vg + (int64_t)(cx & COL_MASK) * 64 * v_rs); vdone = cur; }
         load_q(r);
-        if (t == g0) FWD_WALL(2);
         while (cur < seg_b) {
           // draw the tile after next; the value is picked up inside the tile
           int drawn = 0;
@@ -650,7 +635,6 @@ void fwd_kernel(const FwdParams prm) {
           cb_nxt = __builtin_amdgcn_readfirstlane(cb_nn_v);
         }  // tiles of this wavefront
       }
-      FWD_WALL(3 + 3 * nseg);
       // ---- merge the wavefronts' results of this row block through LDS ----
       // Each wavefront publishes (m, l) per query and, round by round, R accumulator registers in
       // its own V buffer ([register][lane] floats); in every round each wavefront reduces QPW
@@ -744,7 +728,6 @@ void fwd_kernel(const FwdParams prm) {
           }
           __syncthreads();
         }
-        FWD_WALL(4 + 3 * nseg);
         if (full) {
           if (w == 0 && g == 0 && prm.lse != nullptr) {
 #pragma unroll
@@ -869,8 +852,6 @@ void fwd_kernel(const FwdParams prm) {
           }
         }
       }
-      FWD_WALL(5 + 3 * nseg);
-      ++nseg;
       t = seg_b;
       ++r;
     }
@@ -934,8 +915,6 @@ static size_t pair_parts_bytes(int B, int H, int N, int D, int split) {
   return split > 1 ? (size_t)split * B * H * N * (D + 2) * sizeof(float) : 0;
 }
 
-static int quad_slots_of_device() { return 2 * compute_units(); }   // two wavefront groups per workgroup, one workgroup per compute unit
-
 size_t coop_workspace_bytes(int B, int H, int N, int D) {
   if (D == 256) return 256 + pair_parts_bytes(B, H, N, D, pair_split(B, H, N / 64, D));   // the pair kernel only
   const int nb = N / 64;
@@ -943,15 +922,10 @@ size_t coop_workspace_bytes(int B, int H, int N, int D) {
   return slots_bytes(B, H, W, D) + (size_t)B * H * nb * sizeof(unsigned long long);
 }
 
-// one size for bsattn_fwd, bsattn_fwd_elementwise and bsattn_fwd_quads
-size_t fwd_workspace_bytes(int B, int H, int N, int D) {
-  const size_t coop = coop_workspace_bytes(B, H, N, D);
-  const size_t quad = D == 64 ? quad_workspace_bytes(quad_slots_of_device(), B, H, N / 64) : 0;
-  return coop > quad ? coop : quad;
-}
+// one size for bsattn_fwd and bsattn_fwd_elementwise
+size_t fwd_workspace_bytes(int B, int H, int N, int D) { return coop_workspace_bytes(B, H, N, D); }
 
 void launch_fwd_pair(const FwdParams& prm, int D, int dt, bool elementwise, hipStream_t st);   // attn_fwd_pair.hip
-void launch_fwd_quad(const FwdParams& prm, int dt, hipStream_t st);                            // attn_fwd_quad.hip
 // D = 128 with enough row blocks in the launch to fill the chip goes to the kernel that gives each
 // row block to one wavefront pair (two wavefronts per SIMD, no merges between workgroups).  With
 // fewer row blocks its critical path is the longest row, which the host cannot see (the lists
@@ -1053,9 +1027,6 @@ int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
     prm.perm_fast = F;
     prm.perm_min_tiles = (int)((int64_t)prm.nb * prm.nb * 3 / 4);
   }
-#ifdef FWD_TIMELINE
-  prm.part_o = getenv("BSATTN_FWD_TIMELINE") ? (float*)strtoull(getenv("BSATTN_FWD_TIMELINE"), nullptr, 16) : nullptr;
-#endif
   prm.out_f32 = s.out_dtype == BSATTN_F32;
   prm.qk_scale = s.sm_scale * 1.4426950408889634f;
   for (int i = 0; i < 3; ++i) { prm.qs[i] = s.qs[i]; prm.ks[i] = s.ks[i]; prm.vs[i] = s.vs[i]; prm.os[i] = s.os[i]; }
@@ -1082,29 +1053,6 @@ int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
     if (s.D == 64) { if (dt == 0) launch_fwd_t<64, 0, true>(prm, BH, st); else if (dt == 1) launch_fwd_t<64, 1, true>(prm, BH, st); else launch_fwd_t<64, 2, true>(prm, BH, st); }
     else { if (dt == 0) launch_fwd_t<128, 0, true>(prm, BH, st); else if (dt == 1) launch_fwd_t<128, 1, true>(prm, BH, st); else launch_fwd_t<128, 2, true>(prm, BH, st); }
   }
-  return launch_status();
-}
-
-// Forward over quad lists (attn_fwd_quad.hip): head dimension 64, block masks.
-int launch_fwd_quads(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* row_ptr,
-                     const int32_t* quad_ptr, const int32_t* quad_list, const AttnShape& s, void* ws, hipStream_t st) {
-  FwdParams prm = {};
-  prm.q = q; prm.k = k; prm.v = v; prm.o = o; prm.lse = lse;
-  prm.row_ptr = row_ptr; prm.quad_ptr = quad_ptr; prm.quad_list = quad_list; prm.ws = (float*)ws;
-  prm.perm_n = 0; prm.perm_fast = 0; prm.perm_min_tiles = 0;
-  prm.B = s.B; prm.H = s.H; prm.N = s.N; prm.nb = s.N / 64; prm.Bm = s.Bm; prm.Hm = s.Hm;
-  prm.epoch = next_epoch();
-  prm.out_f32 = s.out_dtype == BSATTN_F32;
-  prm.qk_scale = s.sm_scale * 1.4426950408889634f;
-  for (int i = 0; i < 3; ++i) { prm.qs[i] = s.qs[i]; prm.ks[i] = s.ks[i]; prm.vs[i] = s.vs[i]; prm.os[i] = s.os[i]; }
-  prm.qslots = quad_slots_of_device();
-  prm.qcounters = (unsigned long long*)((char*)ws + quad_parts_bytes(prm.qslots));
-  prm.vt = (const unsigned short*)((char*)prm.qcounters + quad_counters_bytes(s.B, s.H, prm.nb));
-#ifdef QUAD_TIMELINE
-  prm.part_o = getenv("BSATTN_QUAD_TIMELINE") ? (float*)strtoull(getenv("BSATTN_QUAD_TIMELINE"), nullptr, 16) : nullptr;
-#endif
-  const bool bf = s.dtype == BSATTN_BF16;
-  launch_fwd_quad(prm, !bf ? 0 : (prm.out_f32 ? 1 : 2), st);
   return launch_status();
 }
 

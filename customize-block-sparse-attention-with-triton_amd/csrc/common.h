@@ -5,7 +5,7 @@
 #include <atomic>
 #include "bsattn.h"
 
-#define BSATTN_VERSION 100
+#define BSATTN_VERSION BSATTN_ABI_VERSION
 
 namespace bsattn {
 
@@ -16,8 +16,6 @@ int launch_block_mask_to_lists(const uint8_t* block, int Bm, int Hm, int nb, int
                                int64_t sm, int64_t sn, int32_t* row_ptr, int32_t* col_idx,
                                int32_t* groups, int32_t* counts, int32_t* ws, hipStream_t st);
 
-int launch_quad_lists(const int32_t* row_ptr, const int32_t* col_idx, int Bm, int Hm, int nb, int32_t* quad_ptr,
-                      int32_t* quad_list, int32_t* stats, hipStream_t st);
 int launch_tail_tiles(int Bm, int Hm, int nb, int valid, int transpose, const int32_t* row_ptr,
                       const int32_t* col_idx, uint8_t* partial, unsigned long long* bits, hipStream_t st);
 int launch_reduce_pack(const uint8_t* dense, int Bm, int Hm, int N, int64_t sb, int64_t sh, int64_t sm,
@@ -59,14 +57,6 @@ int get_deterministic();
 int launch_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                const int32_t* row_ptr, const int32_t* col_idx, const uint8_t* tile_partial,
                const uint64_t* tile_bits, const AttnShape& s, void* ws, hipStream_t st);
-int launch_fwd_quads(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* row_ptr,
-                     const int32_t* quad_ptr, const int32_t* quad_list, const AttnShape& s, void* ws, hipStream_t st);
-// attn_fwd_quad.hip: the forward kernel for head dimension 64 that shares K/V tiles between the four
-// row blocks of a quad (fast when neighbouring row blocks keep the same column blocks)
-bool quad_supported(const AttnShape& s);
-size_t quad_workspace_bytes(int slots, int B, int H, int nb);
-size_t quad_parts_bytes(int slots);
-size_t quad_counters_bytes(int B, int H, int nb);
 size_t coop_workspace_bytes(int B, int H, int N, int D);   // what launch_fwd itself needs
 // Address, on the current device, of the library's own scratch array (BSATTN_STATIC_SCRATCH_BYTES).
 int static_scratch(void** ptr);

@@ -19,11 +19,6 @@ struct FwdParams {
   float* part_o; float* part_ml;   // split > 1: unnormalised fp32 O parts [split][B*H][N][D] and their (m, l) [split][B*H][N][2]
   int B, H, N, nb, Bm, Hm, W;   // W: workgroups per head
   int first_ids;                // workgroups with a linear id below this are the first on their compute unit
-  const int32_t* quad_ptr;      // quad kernel: prefix sums of the sizes of the quads' union lists
-  const int32_t* quad_list;     // quad kernel: the union lists, nb entries apart (column block | membership << 16)
-  const unsigned short* vt;     // quad kernel: V transposed, [B*H][64][N] (vt_kernel)
-  int qslots;                   // quad kernel: wavefront groups of the launch (two per workgroup)
-  unsigned long long* qcounters;   // quad kernel: per row block, parts that have arrived (tagged with `epoch`)
   int out_f32;
   float qk_scale;  // sm_scale * log2(e)
   int64_t qs[3], ks[3], vs[3], os[3];

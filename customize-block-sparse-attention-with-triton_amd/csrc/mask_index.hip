@@ -227,93 +227,6 @@ __global__ __launch_bounds__(1024) void count_scan_kernel(const uint8_t* __restr
 
 
 // ---------------------------------------------------------------------------------------
-// Quad lists: four consecutive row blocks of a mask head form a quad; the forward kernel for
-// masks with similar neighbouring rows walks, per quad, the union of the four column lists.
-// One wavefront per quad: the four lists are ORed into bitmaps in LDS (at most 2048 column blocks),
-// entry i of the union goes to quad_list[quad * nb + i] = column block | membership of the four
-// rows << 16, the union's size to quad_ptr[quad + 1] (turned into prefix sums by scan_quads_kernel).
-// ---------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void quad_union_kernel(const int32_t* __restrict__ row_ptr,
-                                                         const int32_t* __restrict__ col_idx, int quads,
-                                                         int nb, int nq, int32_t* __restrict__ quad_ptr,
-                                                         int32_t* __restrict__ quad_list) {
-  __shared__ unsigned bitmap_all[4][4][64];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int qid = blockIdx.x * 4 + wave;
-  if (qid >= quads) return;
-  unsigned (*bitmap)[64] = bitmap_all[wave];
-  const int mh = qid / nq, qi = qid - mh * nq;
-  const int32_t* rp = row_ptr + (int64_t)mh * nb;
-#pragma unroll
-  for (int rr = 0; rr < 4; ++rr) bitmap[rr][lane] = 0u;
-#pragma unroll
-  for (int rr = 0; rr < 4; ++rr) {
-    const int row = 4 * qi + rr;
-    if (row >= nb) break;
-    const int a = rp[row], b = rp[row + 1];
-    for (int t = a + lane; t < b; t += 64) {
-      const int c = col_idx[t];
-      atomicOr(&bitmap[rr][c >> 5], 1u << (c & 31));
-    }
-  }
-  // (the LDS operations of one wavefront complete in order: the reads below see the ORs above)
-  unsigned m[4];
-#pragma unroll
-  for (int rr = 0; rr < 4; ++rr) m[rr] = bitmap[rr][lane];
-  unsigned un = m[0] | m[1] | m[2] | m[3];
-  const int cnt = __popc(un);
-  int incl = cnt;
-#pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    const int o = __shfl_up(incl, off);
-    if (lane >= off) incl += o;
-  }
-  int32_t* dst = quad_list + (int64_t)qid * nb + (incl - cnt);
-  while (un != 0u) {
-    const int bit = __builtin_ctz(un);
-    un &= un - 1u;
-    const unsigned memb = ((m[0] >> bit) & 1u) | (((m[1] >> bit) & 1u) << 1) | (((m[2] >> bit) & 1u) << 2) |
-                          (((m[3] >> bit) & 1u) << 3);
-    *dst++ = (lane * 32 + bit) | (int)(memb << 16);
-  }
-  if (lane == 63) quad_ptr[qid + 1] = incl;
-}
-
-// single workgroup: quad_ptr[1 .. quads] (sizes) -> inclusive prefix sums in place, quad_ptr[0] = 0;
-// stats[0] = entries of all unions, stats[1] = kept tiles of the mask (row_ptr[rows])
-__global__ __launch_bounds__(1024) void scan_quads_kernel(int32_t* __restrict__ quad_ptr, int quads,
-                                                          const int32_t* __restrict__ row_ptr, int rows,
-                                                          int32_t* __restrict__ stats) {
-  __shared__ int s_t[1024];
-  const int tid = threadIdx.x;
-  const int per = (quads + 1023) / 1024;
-  const int q0 = min(quads, tid * per), q1 = min(quads, q0 + per);
-  int t = 0;
-  for (int q = q0; q < q1; ++q) t += quad_ptr[q + 1];
-  s_t[tid] = t;
-  __syncthreads();
-  for (int off = 1; off < 1024; off <<= 1) {
-    int at = 0;
-    if (tid >= off) at = s_t[tid - off];
-    __syncthreads();
-    s_t[tid] += at;
-    __syncthreads();
-  }
-  int run = s_t[tid] - t;
-  for (int q = q0; q < q1; ++q) { run += quad_ptr[q + 1]; quad_ptr[q + 1] = run; }
-  if (tid == 0) quad_ptr[0] = 0;
-  if (tid == 1023) { stats[0] = s_t[1023]; stats[1] = row_ptr[rows]; }
-}
-
-int launch_quad_lists(const int32_t* row_ptr, const int32_t* col_idx, int Bm, int Hm, int nb, int32_t* quad_ptr,
-                      int32_t* quad_list, int32_t* stats, hipStream_t st) {
-  const int nq = (nb + 3) / 4, quads = Bm * Hm * nq;
-  hipLaunchKernelGGL(quad_union_kernel, dim3((quads + 3) / 4), dim3(256), 0, st, row_ptr, col_idx, quads, nb, nq,
-                     quad_ptr, quad_list);
-  hipLaunchKernelGGL(scan_quads_kernel, dim3(1), dim3(1024), 0, st, quad_ptr, quads, row_ptr, Bm * Hm * nb, stats);
-  return launch_status();
-}
-
 // The 64 x 64 bit matrix whose row r is the word of lane r, transposed: six rounds of block swaps between lanes
 // l and l ^ j (j = 32 ... 1), each exchanging the off-diagonal j x j blocks of every 2j x 2j block.
 __device__ __forceinline__ unsigned long long transpose64(unsigned long long word, int lane) {

@@ -32,9 +32,6 @@ _SIGNATURES = {
     "bsattn_fwd_workspace": ([_i, _i, _i, _i, ctypes.POINTER(ctypes.c_size_t)], _i),
     "bsattn_fwd": ([_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f,
                     _p, _p, _p, _p, _p, ctypes.c_size_t, _p], _i),
-    "bsattn_quad_lists": ([_p, _p, _i, _i, _i, _p, _p, _p, _p], _i),
-    "bsattn_fwd_quads": ([_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f,
-                          _p, _p, _p, _p, _p, ctypes.c_size_t, _p], _i),
     "bsattn_fwd_static": ([_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f,
                            _p, _p, _p, _p, _p], _i),
     "bsattn_fwd_elementwise": ([_p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f,
@@ -45,6 +42,7 @@ _SIGNATURES = {
     "bsattn_reorder": ([_p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p], _i),
 }
 EXPORTS = tuple(_SIGNATURES)
+ABI_MAJOR = 2      # BSATTN_ABI_VERSION / 100 of the header these signatures were written against
 
 
 def lib():
@@ -59,6 +57,9 @@ def lib():
             fn = getattr(l, name)
             fn.argtypes = argtypes
             fn.restype = restype
+        if l.bsattn_version() // 100 != ABI_MAJOR:
+            raise RuntimeError("%s has ABI version %d, this package needs %d.x: rebuild it with build.py"
+                               % (LIB_PATH, l.bsattn_version(), ABI_MAJOR))
         _lib = l
     return _lib
 

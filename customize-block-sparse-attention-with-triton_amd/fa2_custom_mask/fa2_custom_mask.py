@@ -4,13 +4,13 @@ Mirrors fa2_custom_mask/fa2_custom_mask.py of the reference: `build_groups_from_
 (:15-38) and the autograd function behind `flash_attention_custom_mask` (:40-157), with the
 device work done by hand-written gfx950 kernels reached through the C ABI in include/bsattn.h.
 """
+import collections
 import ctypes
 
 import torch
 
 from . import _ext
-from .utils import (TILE, QUAD_MAX_BLOCKS, QUAD_MAX_QUADS, block_mask_to_lists, mask_to_lists, num_tiles,
-                    is_block_form, _check_mask)
+from .utils import TILE, block_mask_to_lists, mask_to_lists, num_tiles, is_block_form, _check_mask
 
 
 def build_groups_from_block_mask(mask):
@@ -34,20 +34,38 @@ def _prep(x):
     return x
 
 
-_workspaces = {}
+_workspaces = collections.OrderedDict()
+WORKSPACE_CACHE_STREAMS = 8          # (device, stream) pairs whose workspace is kept
+WORKSPACE_CACHE_BYTES = 256 << 20    # a larger workspace serves its call and is then given back
+
+
+def clear_workspaces():
+    """Gives back the workspaces kept for reuse."""
+    _workspaces.clear()
 
 
 def _workspace(nbytes, device):
     """Scratch memory for one call, kept per (device, stream) and reused by the next call on that stream:
     the kernels need no particular contents on entry, and calls on one stream run one after the
-    other.  (Plans own their workspaces: they may be replayed from graphs on any stream.)"""
+    other.  The cache is bounded (the least recently used stream's workspace goes first, a workspace above
+    WORKSPACE_CACHE_BYTES is not kept), and nothing is kept or taken from it while a graph is being captured:
+    memory first allocated under capture belongs to the graph's pool.  (Plans own their workspaces: they may be
+    replayed from graphs on any stream.)"""
     stream = torch.cuda.current_stream(device)
+    handle = ctypes.c_void_p(stream.cuda_stream)
+    if torch.cuda.is_current_stream_capturing():
+        return torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device), handle
     key = (device.index, stream.cuda_stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
-    return ws, ctypes.c_void_p(stream.cuda_stream)
+        if nbytes <= WORKSPACE_CACHE_BYTES:
+            _workspaces[key] = ws
+            while len(_workspaces) > WORKSPACE_CACHE_STREAMS:
+                _workspaces.popitem(last=False)
+    if key in _workspaces:
+        _workspaces.move_to_end(key)
+    return ws, handle
 
 
 def _like(x, dtype):
@@ -114,37 +132,6 @@ def set_deterministic(on):
     return bool(_ext.lib().bsattn_set_deterministic(1 if on else 0))
 
 
-QUAD_MIN_EFFICIENCY = 0.7
-# The kernel that walks quads is chosen by the caller (ForwardPlan(quads=True), or this switch for the
-# autograd path): at the sizes measured so far the kernel behind bsattn_fwd is the faster of the two.
-QUAD_AUTO = False
-
-
-def _use_quads(lists, B, H, N, D, wait=False):
-    """Whether the forward goes to the kernel that walks quads (bsattn_fwd_quads): head dimension 64,
-    a block mask it can index, and row blocks that agree with their neighbours.  The last is a
-    property of the mask's content, which lives on the device: it is known from the statistics the
-    quad preprocessing sends to the host, and until they have arrived (first call after a new mask,
-    unless wait=True) the answer is no."""
-    nb = N // TILE
-    if not QUAD_AUTO and not wait:
-        return False
-    if D != 64 or N % TILE or lists.bits is not None or nb > QUAD_MAX_BLOCKS or nb < 4:
-        return False
-    shared = (lists.Bm, lists.Hm) == (1, 1)
-    if not shared and (lists.Bm, lists.Hm) != (B, H):
-        return False
-    if ((nb + 3) // 4) * (1 if shared else B * H) > QUAD_MAX_QUADS:
-        return False
-    # the quad form is only made for lists that are used again (a mask that changes with every call
-    # would pay the preprocessing each time)
-    lists.uses += 1
-    if lists.uses < 2 and not wait:
-        return False
-    eff = lists.quads().efficiency(wait)
-    return eff is not None and eff >= QUAD_MIN_EFFICIENCY
-
-
 def _forward(q, k, v, lists, sm_scale, out_dtype, want_lse):
     B, H, N, D = q.shape
     q, k, v = _prep(q), _prep(k), _prep(v)
@@ -157,10 +144,7 @@ def _forward(q, k, v, lists, sm_scale, out_dtype, want_lse):
               ws.data_ptr(), wsb, stream)
     ptrs = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr() if want_lse else None,
             lists.row_ptr.data_ptr(), lists.col_idx.data_ptr())
-    if _use_quads(lists, B, H, N, D):
-        qd = lists.quads()
-        rc = _ext.lib().bsattn_fwd_quads(*ptrs[:6], qd.quad_ptr.data_ptr(), qd.quad_list.data_ptr(), *common)
-    elif lists.bits is None:
+    if lists.bits is None:
         rc = _ext.lib().bsattn_fwd(*ptrs, *common)
     else:                                      # elementwise mask: exact inside partly set tiles
         rc = _ext.lib().bsattn_fwd_elementwise(*ptrs, lists.partial.data_ptr(), lists.bits.data_ptr(), *common)
@@ -172,10 +156,7 @@ class ForwardPlan:
     """A forward call with every buffer allocated and every C argument marshalled once; run()
     only enqueues the kernels.  For loops that repeat the same shapes (serving, benchmarks)."""
 
-    def __init__(self, q, k, v, lists, sm_scale, out_dtype=None, stream=None, quads=None):
-        """quads: True / False forces the kernel that walks quads on or off; None follows QUAD_AUTO
-        (off unless set; when set, decided from the mask, which waits for the mask's statistics: a
-        plan is set-up work)."""
+    def __init__(self, q, k, v, lists, sm_scale, out_dtype=None, stream=None):
         B, H, N, D = q.shape
         if N % TILE or D not in (64, 128, 256):
             raise ValueError("a plan takes whole tiles only: N % 64 == 0 and D in {64, 128, 256}")
@@ -191,17 +172,10 @@ class ForwardPlan:
                 float(sm_scale)) + self._keep + (self.ws.data_ptr(), wsb, ctypes.c_void_p(stream.cuda_stream))
         head = (self.q.data_ptr(), self.k.data_ptr(), self.v.data_ptr(), self.o.data_ptr(), self.lse.data_ptr(),
                 lists.row_ptr.data_ptr())
-        use_quads = (QUAD_AUTO and _use_quads(lists, B, H, N, D, wait=True)) if quads is None else quads
         if lists.bits is not None:
             raise ValueError("a plan takes block masks only")
-        if use_quads:
-            qd = lists.quads()
-            self._args = head + (qd.quad_ptr.data_ptr(), qd.quad_list.data_ptr()) + tail
-            self._fn = _ext.lib().bsattn_fwd_quads
-        else:
-            self._args = head + (lists.col_idx.data_ptr(),) + tail
-            self._fn = _ext.lib().bsattn_fwd
-        self.uses_quads = use_quads
+        self._args = head + (lists.col_idx.data_ptr(),) + tail
+        self._fn = _ext.lib().bsattn_fwd
 
     def run(self):
         rc = self._fn(*self._args)

@@ -29,63 +29,13 @@ class TileLists:
     entries valid), counts int32 [2] = (G, T), groups int32 [Bm*Hm*nb, 5] (first G rows
     valid) or None."""
 
-    __slots__ = ("row_ptr", "col_idx", "groups", "counts", "Bm", "Hm", "nb", "partial", "bits", "_quads", "uses")
+    __slots__ = ("row_ptr", "col_idx", "groups", "counts", "Bm", "Hm", "nb", "partial", "bits")
 
     def __init__(self, row_ptr, col_idx, groups, counts, Bm, Hm, nb):
         self.row_ptr, self.col_idx, self.groups, self.counts = row_ptr, col_idx, groups, counts
         self.Bm, self.Hm, self.nb = Bm, Hm, nb
         # elementwise masks only: per kept tile "partly set" flag and packed 64 x 64 bits
         self.partial, self.bits = None, None
-        self._quads = None
-        self.uses = 0          # forward calls that have looked at these lists
-
-    def quads(self):
-        """The quad form of the lists (QuadLists), built on first use."""
-        if self._quads is None:
-            self._quads = QuadLists(self)
-        return self._quads
-
-
-QUAD_MAX_BLOCKS = 2048      # BSATTN_QUAD_MAX_BLOCKS
-QUAD_MAX_QUADS = 4096       # quads per launch (per head for a mask shared by all heads)
-
-
-class QuadLists:
-    """Union lists of the quads (four consecutive row blocks) of a block mask, for the forward kernel
-    that shares K/V tiles between the row blocks of a quad: quad_ptr int32 [quads+1], quad_list int32
-    [quads*nb] (column block | membership << 16), quad_stats int32 [2] = (entries of all unions, kept
-    tiles).  The two statistics are also copied to the host without synchronising: efficiency()
-    answers once the copy has arrived."""
-
-    __slots__ = ("quad_ptr", "quad_list", "quad_stats", "_host", "_event", "_eff")
-
-    def __init__(self, lists):
-        dev = lists.row_ptr.device
-        quads = lists.Bm * lists.Hm * ((lists.nb + 3) // 4)
-        self.quad_ptr = torch.empty(quads + 1, dtype=torch.int32, device=dev)
-        self.quad_list = torch.empty(quads * lists.nb, dtype=torch.int32, device=dev)
-        self.quad_stats = torch.empty(2, dtype=torch.int32, device=dev)
-        rc = _ext.lib().bsattn_quad_lists(lists.row_ptr.data_ptr(), lists.col_idx.data_ptr(), lists.Bm, lists.Hm,
-                                          lists.nb, self.quad_ptr.data_ptr(), self.quad_list.data_ptr(),
-                                          self.quad_stats.data_ptr(), _ext.current_stream(dev))
-        _ext.check(rc, "bsattn_quad_lists")
-        self._host = torch.empty(2, dtype=torch.int32, pin_memory=True)
-        self._host.copy_(self.quad_stats, non_blocking=True)
-        self._event = torch.cuda.Event()
-        self._event.record(torch.cuda.current_stream(dev))
-        self._eff = None
-
-    def efficiency(self, wait=False):
-        """Kept tiles / tile slots of the walk over the unions (1.0: the four lists of every quad agree);
-        None while the statistics have not reached the host (wait=True synchronises on them)."""
-        if self._eff is None:
-            if wait:
-                self._event.synchronize()
-            elif not self._event.query():
-                return None
-            union, kept = self._host.tolist()
-            self._eff = kept / (4.0 * union) if union > 0 else 0.0
-        return self._eff
 
 
 def _check_mask(mask):

@@ -48,6 +48,13 @@ extern "C" {
 #define BSATTN_BF16 1
 #define BSATTN_F32 2 /* outputs only */
 
+/* ABI version of the library, major * 100 + minor.  The major number changes whenever an entry point's
+ * argument list changes or an entry point goes away; a caller built against this header checks
+ * bsattn_version() / 100 == BSATTN_ABI_VERSION / 100 before its first other call.
+ *   100: first layout.
+ *   200: bsattn_bwd and bsattn_bwd_elementwise take dq_strides, dk_strides, dv_strides after
+ *        do_strides; the entry points of the forward over quads of row blocks are gone. */
+#define BSATTN_ABI_VERSION 200
 int bsattn_version(void);
 /* Process-wide switch (default off), returns the previous setting.  On: the forward's result
  * depends on nothing but its inputs and the device (two runs give the same bits).  Off: the
@@ -92,22 +99,6 @@ int bsattn_block_mask_to_lists(const uint8_t* block, int Bm, int Hm, int nb,
                                int32_t* row_ptr, int32_t* col_idx, int32_t* groups,
                                int32_t* counts, void* workspace, size_t workspace_bytes,
                                void* stream);
-
-/* Quad lists: a second form of the kept-tile lists, for bsattn_fwd_quads.  Four consecutive row
- * blocks of a mask head form a quad (the last quad of a head may hold fewer).  For quad j
- * (j = mask head * ceil(nb/4) + index within the head):
- *   quad_list[j*nb + i], i < size_j: the i-th column block, ascending, that any row block of the quad
- *       keeps, in bits 0..15, and in bits 16..19 which of the quad's row blocks keep it;
- *   quad_ptr  int32 [Bm*Hm*ceil(nb/4) + 1]: exclusive prefix sums of size_j;
- *   quad_stats int32 [2]: sum of all size_j, and the number of kept tiles of the mask.  Walking the
- *       unions costs 4 * quad_stats[0] tile slots for quad_stats[1] kept tiles: the closer the
- *       ratio quad_stats[1] / (4 * quad_stats[0]) is to 1, the better bsattn_fwd_quads does.
- * row_ptr / col_idx as made by bsattn_block_mask_to_lists for the same [Bm,Hm,nb,nb] mask;
- * quad_list has capacity Bm*Hm*ceil(nb/4)*nb; nb <= BSATTN_QUAD_MAX_BLOCKS.  No counterpart in the
- * reference, whose kernel walks one row list per program (fa2_custom_mask/fa2_fwd.py:152-153). */
-#define BSATTN_QUAD_MAX_BLOCKS 2048
-int bsattn_quad_lists(const int32_t* row_ptr, const int32_t* col_idx, int Bm, int Hm, int nb,
-                      int32_t* quad_ptr, int32_t* quad_list, int32_t* quad_stats, void* stream);
 
 /* ------------------------------------------------------------------------------------
  * Elementwise masks (exact semantics inside partly set tiles: the naive masked_fill(-inf)
@@ -176,33 +167,29 @@ int bsattn_fwd_workspace(int B, int H, int N, int D, size_t* bytes);
  * A row block whose kept tiles are split over several workgroups is finished by the workgroup
  * that completes its share last (parts and one counter per row block live in the workspace):
  * no workgroup ever waits for another, so the call completes whatever else runs on the GPU
- * and however many workgroups are resident at a time.  The workspace needs no initialisation
+ * and however many workgroups are resident at a time.  The workspace (16-byte aligned, else
+ * BSATTN_ERR_STRIDE: it holds 64-bit counters behind the parts) needs no initialisation
  * and may be reused by the next call on the same stream; two calls that overlap in time need
- * two workspaces. */
+ * two workspaces.
+ * Memory ordering of that hand-off.  A holder of a part writes it with device-scope stores (they
+ * are served by the memory all compute units share, never by a cache only some of them see), waits
+ * until every one of them has been acknowledged (s_waitcnt vmcnt(0) in each wavefront, then the
+ * workgroup barrier), and only then does one thread count the part in with a compare-and-swap on
+ * the row block's counter.  The workgroup that finds all other parts counted reads them with
+ * device-scope loads issued after its compare-and-swap has returned (the value is passed through
+ * LDS and a barrier to the other wavefronts, so no load of a part can be issued before it).  Each
+ * part was complete in shared memory before its count became visible, and the reader's loads
+ * cannot be served from a stale cache line, so the counter update itself is relaxed: release /
+ * acquire order on it would add a write-back and an invalidation of a whole L2 for accesses that
+ * are already ordered, measured at 9 us per launch (N = 17536, one head, keep 0.1: 31 -> 41 us).
+ * A counter holds (launch mark << 16 | parts counted): contents left by earlier launches carry
+ * another mark and read as zero, and the last arriver puts the counter back to zero. */
 int bsattn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                const int32_t* row_ptr, const int32_t* col_idx, int Bm, int Hm,
                int B, int H, int N, int D, int dtype, int out_dtype, float sm_scale,
                const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
                const int64_t* o_strides, void* workspace, size_t workspace_bytes,
                void* stream);
-
-/* The same forward (same arguments, same results up to rounding) by a kernel made for masks whose
- * neighbouring row blocks keep nearly the same column blocks: dense, block-causal, banded, frame-wise
- * masks.  The four row blocks of a quad walk the union of their column lists together and share
- * every K and V tile, so a launch computes on 4 * quad_stats[0] tile slots instead of
- * quad_stats[1] tiles (see bsattn_quad_lists): at a ratio near 1 it is the faster entry point, for
- * scattered masks bsattn_fwd is.  Replaces the same reference launch as bsattn_fwd
- * (fa2_custom_mask/fa2_custom_mask.py:69-87).  Head dimension 64 only (BSATTN_ERR_HEAD_DIM);
- * N <= 64 * BSATTN_QUAD_MAX_BLOCKS, (Bm, Hm) = (1, 1) or (B, H), and at most 4096 quads in the
- * launch (per head for a shared mask): BSATTN_ERR_RANGE otherwise.  Workspace as bsattn_fwd
- * (bsattn_fwd_workspace bytes).  Row blocks shared between workgroups are finished by the
- * workgroup that arrives last (a counter per row block in the workspace, no waiting). */
-int bsattn_fwd_quads(const void* q, const void* k, const void* v, void* o, float* lse,
-                     const int32_t* row_ptr, const int32_t* quad_ptr, const int32_t* quad_list,
-                     int Bm, int Hm, int B, int H, int N, int D, int dtype, int out_dtype,
-                     float sm_scale, const int64_t* q_strides, const int64_t* k_strides,
-                     const int64_t* v_strides, const int64_t* o_strides, void* workspace,
-                     size_t workspace_bytes, void* stream);
 
 /* Forward that allocates nothing and needs no workspace argument.  It has no counterpart in the
  * reference; it is for callers that cannot allocate device memory around the call: code under HIP
@@ -248,7 +235,8 @@ int bsattn_fwd_elementwise(const void* q, const void* k, const void* v, void* o,
 
 /* Bytes of workspace bsattn_bwd needs: delta = rowsum(O * dO), and for launches with few row
  * blocks the fp32 parts of dQ, dK, dV of row / column lists walked by several workgroups.
- * Depends on the shape and on the number of compute units of the current device. */
+ * Depends on the shape and on the number of compute units of the current device.  The workspace
+ * must be 16-byte aligned (BSATTN_ERR_STRIDE otherwise). */
 int bsattn_bwd_workspace(int B, int H, int N, int D, size_t* bytes);
 
 /* q,k,v,o,d_o: [B,H,N,D] fp16/bf16 with their own strides; lse from bsattn_fwd.

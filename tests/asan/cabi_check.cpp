@@ -43,10 +43,6 @@ int main() {
   EXPECT(bsattn_mask_lists_workspace(64, 64, 4096, &n), BSATTN_ERR_RANGE);
   EXPECT(bsattn_fwd_static(P, P, P, P, nullptr, (const int32_t*)P, (const int32_t*)P, 1, 1, 1, 1, 17536, 256, 0, 0, 0.1f, ok, ok, ok,
                            ok, nullptr), BSATTN_ERR_STATIC_LIMIT);
-  EXPECT(bsattn_quad_lists((const int32_t*)P, (const int32_t*)P, 1, 1, 4096, (int32_t*)P, (int32_t*)P, (int32_t*)P, nullptr),
-         BSATTN_ERR_RANGE);
-  EXPECT(bsattn_fwd_quads(P, P, P, P, nullptr, (const int32_t*)P, (const int32_t*)P, (const int32_t*)P, 1, 1, 1, 1, 256, 128, 0, 0,
-                          0.1f, ok, ok, ok, ok, P, big, nullptr), BSATTN_ERR_HEAD_DIM);
   EXPECT(bsattn_bwd(P, P, P, P, P, (const float*)P, P, P, nullptr, (const int32_t*)P, (const int32_t*)P, (const int32_t*)P,
                     (const int32_t*)P, 1, 1, 1, 1, 64, 64, 0, 0, 0.1f, ok, ok, ok, ok, ok, nullptr, nullptr, nullptr, P, big,
                     nullptr), BSATTN_ERR_NULL);

@@ -1,6 +1,5 @@
 """Host code under the address and undefined-behaviour sanitizers (tests/asan/Makefile, target `asan`): the C
-oracle, the work split of the forward kernel that walks quads (plain integer arithmetic shared with the
-kernel), the range permutation of the forward kernel, and the argument validation of the C ABI.  Needs no GPU; any finding aborts a program."""
+oracle, the range permutation of the forward kernel, and the argument validation of the C ABI.  Needs no GPU; any finding aborts a program."""
 import os
 import subprocess
 
@@ -11,4 +10,4 @@ def test_make_asan(tmp_path):
     out = subprocess.run(["make", "-C", os.path.join(ROOT, "tests", "asan"), "asan", "OUT=" + str(tmp_path)],
                          capture_output=True, text=True)
     assert out.returncode == 0, out.stdout[-3000:] + out.stderr[-3000:]
-    assert out.stdout.count("\nok") >= 4
+    assert out.stdout.count("\nok") >= 3

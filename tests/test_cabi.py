@@ -17,7 +17,8 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_ext.LIB_PATH)
     for name in declared:
         assert getattr(lib, name) is not None
-    assert _ext.lib().bsattn_version() >= 100
+    assert _ext.lib().bsattn_version() // 100 == _ext.ABI_MAJOR
+    assert int(re.search(r"#define BSATTN_ABI_VERSION (\d+)", header).group(1)) == _ext.lib().bsattn_version()
 
 
 def test_strerror():

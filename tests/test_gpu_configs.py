@@ -104,15 +104,33 @@ def test_head_dim_256_row_lists_shared_by_workgroups(dev):
     assert float(np.abs(o[0, 0, 6 * 64:7 * 64]).max()) == 0.0
 
 
-def test_c2_dense_elementwise_mask_n6400(dev):
-    """C2: preprocessing from a dense N x N bool mask (tile-constant) feeds the same result."""
+@pytest.mark.parametrize("keep", [0.1, 1.0])
+@pytest.mark.parametrize("route", ["elementwise", "reduced"])
+def test_c2_dense_elementwise_mask_n6400(dev, keep, route):
+    """C2: the mask arrives as a dense, tile-constant N x N bool tensor (kernel-test.py:18).  Both routes from it
+    (taken as an elementwise mask; reduced to the block mask first) against the oracle on sampled row blocks,
+    and the lists made from the reduced mask against the oracle's, bit for bit."""
     import fa2_custom_mask as fm
     N, nb = 6400, 100
-    block = uniform_block_mask(1, 1, nb, 0.1, 1235)
+    block = uniform_block_mask(1, 1, nb, keep, 1235)
     dense = block.to(dev).repeat_interleave(64, 2).repeat_interleave(64, 3)
-    q, k, v = [x.to(dev) for x in make_qkv(1, 1, N, 64, torch.float16, 1235)]
-    assert same_up_to_rounding(fm.flash_attention_custom_mask(q, k, v, dense, 0.125),
-                               fm.flash_attention_custom_mask(q, k, v, block.to(dev), 0.125))
+    q, k, v = make_qkv(1, 1, N, 64, torch.float16, 1235)
+    sc = 0.125
+    m_in = dense if route == "elementwise" else fm.reduce_dense_mask(dense)
+    if route == "reduced":
+        groups, n_list = fm.build_groups_from_block_mask(m_in)
+        g_ref, n_ref = orc.build_groups_from_block_mask(block.numpy())
+        assert np.array_equal(groups.cpu().numpy(), g_ref) and np.array_equal(n_list.cpu().numpy(), n_ref)
+    o, lse = fm.flash_attention_custom_mask_lse(q.to(dev), k.to(dev), v.to(dev), m_in, sc)
+    o = o.float().cpu().numpy(); lse = lse.cpu().numpy()
+    assert np.isfinite(o).all()
+    qf, kf, vf = f32(q), f32(k), f32(v)
+    for mb in (0, 1, 50, 98, 99):
+        r0, r1 = mb * 64, mb * 64 + 64
+        o_ref, lse_ref = c_oracle.naive_fwd(qf, kf, vf, block.numpy(), sc, r0, r1)
+        d = o[0, 0, r0:r1] - o_ref[0, 0, r0:r1]
+        assert np.abs(d).max() <= 2e-2 and np.linalg.norm(d) / np.linalg.norm(o_ref[0, 0, r0:r1]) <= 1e-3, mb
+        assert np.abs(lse[0, 0, r0:r1] - lse_ref[0, 0, r0:r1]).max() <= 2e-3
 
 
 def test_c5_fwd_bwd_bf16_d128(dev):
@@ -140,42 +158,6 @@ def test_c5_fwd_bwd_bf16_d128(dev):
     for a, b_ in ((o16, o), (dq16, dq), (dk16, dk), (dv16, dv)):
         assert a.dtype == torch.bfloat16
         assert errors(a, b_)[1] <= 3e-3                           # the same values up to bf16 rounding
-
-
-def test_mfma_rate_probe_runs(dev):
-    """The benchmark's measurement aid (a library of its own, not part of the attention library) launches,
-    reports the FLOPs of the launch, leaves the expected sums and a plausible shader clock."""
-    import ctypes
-    import os
-    from fa2_custom_mask import _ext
-    path = os.path.join(os.path.dirname(os.path.dirname(_ext.LIB_PATH)), "probe", "libbsattn_probe.so")
-    lib = ctypes.CDLL(path)
-    lib.probe_mfma_rate.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
-    ops = torch.ones(4096, dtype=torch.float16, device=dev)
-    sink = torch.full((512,), float("nan"), dtype=torch.float32, device=dev)
-    flops = ctypes.c_double()
-    st = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
-    assert lib.probe_mfma_rate(None, 16, sink.data_ptr(), None, st) == -1
-    assert lib.probe_mfma_rate(ops.data_ptr(), 0, sink.data_ptr(), None, st) == -8
-    rc = lib.probe_mfma_rate(ops.data_ptr(), 4, sink.data_ptr(), ctypes.byref(flops), st)
-    assert rc == 0
-    torch.cuda.synchronize()
-    cus = torch.cuda.get_device_properties(dev).multi_processor_count
-    assert flops.value == cus * 8 * 4 * 8 * 2 * 32 * 32 * 16
-    # every accumulator element is 4 iterations x 2 MFMAs per chain x 16 ones = 128; 64 elements per lane
-    assert torch.all(sink[:511] == 128.0 * 64)
-    # the last slot: the shader clock in GHz the first wavefront saw (cycle counter against the 100 MHz wall clock)
-    assert 0.2 < float(sink[511]) < 4.0
-    # the same entry with the forward's softmax instructions beside the MFMAs: 9 MFMAs per iteration
-    lib.probe_mfma_softmax_mix.argtypes = lib.probe_mfma_rate.argtypes
-    g = torch.Generator().manual_seed(3)
-    rnd = torch.randn(4096, generator=g).to(torch.float16).to(dev)
-    sink.fill_(float("nan"))
-    assert lib.probe_mfma_softmax_mix(rnd.data_ptr(), 1 << 21, sink.data_ptr(), None, st) == -8
-    assert lib.probe_mfma_softmax_mix(rnd.data_ptr(), 4, sink.data_ptr(), ctypes.byref(flops), st) == 0
-    torch.cuda.synchronize()
-    assert flops.value == cus * 8 * 4 * 9 * 2 * 32 * 32 * 16
-    assert bool(torch.isfinite(sink).all()) and 0.2 < float(sink[511]) < 4.0
 
 
 def test_committed_toy_fixture(dev):

@@ -32,9 +32,15 @@ def _both(dev, B, H, N, D, dtype, keep, seed):
                 _ext.dtype_code(dtype), float(sc), _ext.strides4(q), _ext.strides4(k), _ext.strides4(v),
                 _ext.strides4(o))
         if static:
-            before = torch.cuda.memory_allocated(dev)
+            # one call first (the library looks up its array's address and sets kernel attributes once per
+            # device); then the free memory of the device itself, which any hipMalloc would lower, not only
+            # torch's own bookkeeping, must be the same before and after a call
+            assert lib.bsattn_fwd_static(*args, st) == 0
+            torch.cuda.synchronize()
+            free_before, before = torch.cuda.mem_get_info(dev)[0], torch.cuda.memory_allocated(dev)
             rc = lib.bsattn_fwd_static(*args, st)
-            assert torch.cuda.memory_allocated(dev) == before
+            torch.cuda.synchronize()
+            assert torch.cuda.mem_get_info(dev)[0] == free_before and torch.cuda.memory_allocated(dev) == before
         else:
             wsb = _ext.fwd_workspace(B, H, N, D)
             ws = torch.empty(wsb, dtype=torch.uint8, device=dev)
@@ -60,6 +66,9 @@ def test_static_forward_matches_workspace_forward(dev):
     _both(dev, 1, 1, 2048, 64, torch.float16, 0.7, 11)
     _both(dev, 1, 2, 512, 64, torch.float16, 0.5, 12)
     _both(dev, 1, 1, 1024, 128, torch.bfloat16, 0.6, 13)
+    # D = 256 with few row blocks: the row lists are shared between workgroups and the scratch array holds
+    # their fp32 parts, which a second kernel sums (2 MB here)
+    _both(dev, 1, 1, 1024, 256, torch.float16, 0.6, 14)
 
 
 def test_static_forward_rejects_shapes_beyond_its_scratch(dev):
