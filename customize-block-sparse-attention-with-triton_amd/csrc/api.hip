@@ -174,6 +174,46 @@ int bsattn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                     sm_scale, q_strides, k_strides, v_strides, o_strides, workspace, workspace_bytes, stream);
 }
 
+// the lists part of bsattn_fwd_block_mask's workspace, rounded up so that the forward's part stays aligned
+static size_t lists_part_bytes(int Bm, int Hm, int nb) {
+  return (((size_t)Bm * Hm * nb * 2 * sizeof(int32_t)) + 255) & ~(size_t)255;
+}
+
+int bsattn_fwd_block_mask_workspace(int Bm, int Hm, int B, int H, int N, int D, size_t* bytes) {
+  if (bytes == nullptr) return BSATTN_ERR_NULL;
+  int rc = check_attn(Bm, Hm, B, H, N, D, BSATTN_F16, BSATTN_F16);
+  if (rc != BSATTN_OK) return rc;
+  size_t lists = 0;
+  if ((rc = bsattn_mask_lists_workspace(Bm, Hm, N / BSATTN_TILE, &lists)) != BSATTN_OK) return rc;
+  *bytes = lists_part_bytes(Bm, Hm, N / BSATTN_TILE) + fwd_workspace_bytes(B, H, N, D);
+  return BSATTN_OK;
+}
+
+int bsattn_fwd_block_mask(const void* q, const void* k, const void* v, void* o, float* lse, const uint8_t* block,
+                          const int64_t* mask_strides, int Bm, int Hm, int32_t* row_ptr, int32_t* col_idx,
+                          int32_t* counts, int B, int H, int N, int D, int dtype, int out_dtype, float sm_scale,
+                          const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                          const int64_t* o_strides, void* workspace, size_t workspace_bytes, void* stream) {
+  if (block == nullptr || mask_strides == nullptr || counts == nullptr) return BSATTN_ERR_NULL;
+  int rc = fwd_check(q, k, v, o, row_ptr, col_idx, Bm, Hm, B, H, N, D, dtype, out_dtype, q_strides, k_strides,
+                     v_strides, o_strides);
+  if (rc != BSATTN_OK) return rc;
+  size_t need = 0;
+  if ((rc = bsattn_fwd_block_mask_workspace(Bm, Hm, B, H, N, D, &need)) != BSATTN_OK) return rc;
+  if (workspace == nullptr || workspace_bytes < need) return BSATTN_ERR_WORKSPACE;
+  if (((uintptr_t)workspace & 15) != 0) return BSATTN_ERR_STRIDE;
+  const int nb = N / BSATTN_TILE;
+  rc = launch_block_mask_to_lists(block, Bm, Hm, nb, mask_strides[0], mask_strides[1], mask_strides[2], mask_strides[3],
+                                  row_ptr, col_idx, nullptr, counts, (int32_t*)workspace, (hipStream_t)stream);
+  if (rc != BSATTN_OK) return rc;
+  AttnShape s;
+  s.B = B; s.H = H; s.N = N; s.D = D; s.Bm = Bm; s.Hm = Hm; s.dtype = dtype; s.out_dtype = out_dtype;
+  s.sm_scale = sm_scale;
+  for (int i = 0; i < 3; ++i) { s.qs[i] = q_strides[i]; s.ks[i] = k_strides[i]; s.vs[i] = v_strides[i]; s.os[i] = o_strides[i]; s.dos[i] = 0; }
+  return launch_fwd(q, k, v, o, lse, row_ptr, col_idx, nullptr, nullptr, s, (char*)workspace + lists_part_bytes(Bm, Hm, nb),
+                    (hipStream_t)stream);
+}
+
 int bsattn_fwd_static(const void* q, const void* k, const void* v, void* o, float* lse,
                       const int32_t* row_ptr, const int32_t* col_idx, int Bm, int Hm, int B, int H, int N,
                       int D, int dtype, int out_dtype, float sm_scale, const int64_t* q_strides,

@@ -91,7 +91,17 @@ void fwd_kernel(const FwdParams prm) {
   #ifndef MIN_TILES
 #define MIN_TILES NW
 #endif
-  const HeadSplit hs = head_split(rp, nb, prm.W, MIN_TILES, prm.first_ids > bh ? (prm.first_ids - bh + BH - 1) / BH : 0);
+  HeadSplit hs = head_split(rp, nb, prm.W, MIN_TILES, prm.first_ids > bh ? (prm.first_ids - bh + BH - 1) / BH : 0, 0);
+  // Long ranges (the regime of the weighted shares) are cut on the axis with gaps and boundaries move to a row
+  // block's end only from very close; short ranges are cut on the plain tile axis and their boundaries move to
+  // the nearer end of a row block from up to SNAP tiles away (row blocks of up to 2 SNAP tiles are never shared).
+#ifndef LONG_GAP
+#define LONG_GAP 8
+#define LONG_SNAP 2
+#endif
+  const bool long_ranges = !ROWS && ((int64_t)hs.T >= (int64_t)EQUAL_SPLIT_BELOW * hs.Peff || hs.Peff >= 3 * nb);   // (or row blocks much longer than the ranges)
+  const int snap = long_ranges ? LONG_SNAP : C::SNAP;
+  if (long_ranges) { hs.gap = LONG_GAP; hs.X = (int64_t)hs.T + (int64_t)LONG_GAP * nb; }
   // Which range this workgroup takes (launches with few heads and long ranges): the ranges of a head start at
   // all phases of a row, and workgroups that share an XCD, hence an L2, get ranges of like phase, so that they
   // walk the same column blocks at the same time (dense N = 17536, one head: 42 instead of 196 MB fetched from
@@ -119,9 +129,11 @@ void fwd_kernel(const FwdParams prm) {
     }
   }
   if (hs.T == 0 || wg >= hs.Peff) return;
-  int g0 = split_begin(hs, wg), g1 = split_begin(hs, wg + 1);
+  // where the range begins and ends on the cutting axis (ROWS: the plain tile axis, as absolute tile offsets)
+  const int64_t x0 = split_pos(hs, wg), x1 = split_pos(hs, wg + 1);
+  int g0 = hs.lo + (int)x0, g1 = hs.lo + (int)x1;     // (ROWS; the other mode finds its tiles below)
   if constexpr (!ROWS) {
-    if (g0 >= g1) return;
+    if (x0 >= x1) return;
   }
 
   unsigned char* lds_k = lds + w * C::WAVE_LDS;
@@ -220,6 +232,7 @@ void fwd_kernel(const FwdParams prm) {
   // FOLD: "-m_i" enters the scores through one extra contraction slice, ones x (-m_hi, -m_lo)
   uintx4 mfrag[2];
   bool fresh = true;
+  int any_m = 0;     // (wave-uniform) some lane's reference exponent is not zero: the extra contraction slice is needed
 
   auto reset_acc = [&]() {
 #pragma unroll
@@ -231,6 +244,7 @@ void fwd_kernel(const FwdParams prm) {
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) { m_i[qb] = 0.f; l_i[qb] = 0.f; mfrag[qb] = uintx4{0u, 0u, 0u, 0u}; }
     fresh = true;
+    any_m = 0;
   };
   auto load_q = [&](int r) {
 #pragma unroll
@@ -284,9 +298,14 @@ void fwd_kernel(const FwdParams prm) {
         s0 = mfma_qk<BF16>(kfr[0][s], qf[qb][s], s0);
         s1 = mfma_qk<BF16>(kfr[1][s], qf[qb][s], s1);
       }
+    };
+    // FOLD: "- m_i" through the extra slice, only while some lane of the wavefront has moved its reference
+    auto mslice = [&](int qb, floatx16& s0, floatx16& s1) {
       if constexpr (FOLD) {
-        s0 = mfma_qk<BF16>(ones_frag, mfrag[qb], s0);
-        s1 = mfma_qk<BF16>(ones_frag, mfrag[qb], s1);
+        if (any_m) {
+          s0 = mfma_qk<BF16>(ones_frag, mfrag[qb], s0);
+          s1 = mfma_qk<BF16>(ones_frag, mfrag[qb], s1);
+        }
       }
     };
     auto read_v = [&]() {
@@ -321,8 +340,11 @@ void fwd_kernel(const FwdParams prm) {
     // finite), some P left the safe fp16 range: recentre() moves m_i to the tile's row maximum
     // and the numerators are redone from the scores, which are still live.
     auto settle = [&](int qb, floatx16& s0, floatx16& s1, float lnew) {
-      if (__any(fresh || (EW && l_i[qb] == 0.f) || !(lnew - l_i[qb] < 16384.0f))) {
+      // (FOLD: the first tile of a row block keeps the reference at 0 when its sums are of moderate size)
+      const bool first = FOLD ? fresh && !(lnew >= 0.25f) : fresh;
+      if (__any(first || (EW && l_i[qb] == 0.f) || !(lnew - l_i[qb] < 16384.0f))) {
         recentre<DB, FOLD, EW>(s0, s1, oacc, qb, qk_scale, m_i[qb], l_i[qb], mfrag[qb], fresh, g);
+        any_m = 1;
         lnew = softmax_tile<FOLD, PB>(s0, s1, qk_scale, m_i[qb], l_i[qb], pf, qb);
       }
       l_i[qb] = lnew;
@@ -354,22 +376,25 @@ void fwd_kernel(const FwdParams prm) {
     };
     // [1]
     scores(0, sa0, sa1);
+    mslice(0, sa0, sa1);
     if constexpr (EW) { if (partial) mask_scores(sa0, sa1, mw0); }
     __builtin_amdgcn_sched_barrier(0);
     // [2]
     scores(1, sb0, sb1);
-    if constexpr (EW) { if (partial) mask_scores(sb0, sb1, mw1); }
     if constexpr (EARLY_V) {
       if (has1) wait_vm<KOPS>(); else wait_vm<0>();  // V(cur) has landed (K(nxt) may be in flight)
       read_v();
     }
     float lnew0 = softmax_tile<FOLD, PB>(sa0, sa1, qk_scale, m_i[0], l_i[0], pf, 0);
+    constexpr int NSC = 2 * KS;
 #pragma unroll
-    for (int it = 0; it < 2 * KS + (FOLD ? 2 : 0); ++it) {
+    for (int it = 0; it < NSC; ++it) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
-      __builtin_amdgcn_sched_group_barrier(0x002, 64 / (2 * KS + (FOLD ? 2 : 0)) + 1, 0);   // its share of the VALU work
+      __builtin_amdgcn_sched_group_barrier(0x002, 64 / NSC + 1, 0);   // its share of the VALU work
     }
     __builtin_amdgcn_sched_barrier(0);
+    mslice(1, sb0, sb1);
+    if constexpr (EW) { if (partial) mask_scores(sb0, sb1, mw1); }
     settle(0, sa0, sa1, lnew0);
     if constexpr (!EARLY_V) {
       if (has1) wait_vm<KOPS>(); else wait_vm<0>();  // V(cur) has landed (K(nxt) may be in flight)
@@ -397,30 +422,35 @@ void fwd_kernel(const FwdParams prm) {
   // ascend, so this is a search; it is done in two rounds of one load per lane (64 evenly spaced
   // entries, then the entries between two of them) instead of a chain of dependent scalar loads.
   // Also returns the entries around x: s = rp[c - 1] (the last one <= x) and e = rp[c] (c <= nb).
-  auto count_le2 = [&](int x0, int x1, int& c0, int& c1, int& s0, int& e0, int& s1, int& e1) {
+  // (The entries are compared as rp[r] + gap * r, their positions on the axis the ranges are cut on, moved by
+  // the head's first tile; gap = 0: plain tile offsets.)
+  auto count_le2 = [&](int64_t x0, int64_t x1, int gap, int& c0, int& c1, int& s0, int& e0, int& s1, int& e1) {
     const int32_t* rpg_ = prm.row_ptr + (int64_t)mh * nb;
     const int step = (nb + 64) / 64;
+    auto key = [&](int i, int v) { return (int64_t)v + (int64_t)gap * i; };
     if (step >= 64) {     // very long sequences: plain binary searches
       int lo = -1, hi = nb + 1;
-      while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (rp[mid] <= x0) lo = mid; else hi = mid; }
+      while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (key(mid, rp[mid]) <= x0) lo = mid; else hi = mid; }
       c0 = hi;
       lo = -1; hi = nb + 1;
-      while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (rp[mid] <= x1) lo = mid; else hi = mid; }
+      while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (key(mid, rp[mid]) <= x1) lo = mid; else hi = mid; }
       c1 = hi;
       s0 = c0 > 0 ? rp[c0 - 1] : 0; e0 = c0 <= nb ? rp[c0] : 0x7fffffff;
       s1 = c1 > 0 ? rp[c1 - 1] : 0; e1 = c1 <= nb ? rp[c1] : 0x7fffffff;
       return;
     }
     const int i1 = lane * step;
-    const int v1 = i1 <= nb ? rpg_[i1] : 0x7fffffff;
-    const int a0 = __builtin_popcountll(__ballot(v1 <= x0)), a1 = __builtin_popcountll(__ballot(v1 <= x1));
+    const bool in1 = i1 <= nb;
+    const int v1 = in1 ? rpg_[i1] : 0x7fffffff;
+    const int a0 = __builtin_popcountll(__ballot(in1 && key(i1, v1) <= x0)), a1 = __builtin_popcountll(__ballot(in1 && key(i1, v1) <= x1));
     const int b0 = (a0 > 0 ? a0 - 1 : 0) * step, b1 = (a1 > 0 ? a1 - 1 : 0) * step;
     const int j0 = b0 + lane, j1 = b1 + lane;
     // (lane `step` holds the next evenly spaced entry, which is > x: it does not count, but may be e)
-    const int w0 = lane <= step && j0 <= nb ? rpg_[j0] : 0x7fffffff;
-    const int w1 = lane <= step && j1 <= nb ? rpg_[j1] : 0x7fffffff;
-    const int k0 = a0 > 0 ? __builtin_popcountll(__ballot(w0 <= x0)) : 0;
-    const int k1 = a1 > 0 ? __builtin_popcountll(__ballot(w1 <= x1)) : 0;
+    const bool in_w0 = lane <= step && j0 <= nb, in_w1 = lane <= step && j1 <= nb;
+    const int w0 = in_w0 ? rpg_[j0] : 0x7fffffff;
+    const int w1 = in_w1 ? rpg_[j1] : 0x7fffffff;
+    const int k0 = a0 > 0 ? __builtin_popcountll(__ballot(in_w0 && key(j0, w0) <= x0)) : 0;
+    const int k1 = a1 > 0 ? __builtin_popcountll(__ballot(in_w1 && key(j1, w1) <= x1)) : 0;
     c0 = b0 + k0;
     c1 = b1 + k1;
     s0 = __builtin_amdgcn_readfirstlane(__shfl(w0, k0 > 0 ? k0 - 1 : 0)); e0 = __builtin_amdgcn_readfirstlane(__shfl(w0, k0));
@@ -526,7 +556,7 @@ void fwd_kernel(const FwdParams prm) {
     {
       // smallest r with rp[r] >= g = number of r with rp[r] <= g - 1 (capped at nb)
       int u0, u1, u2, u3;
-      count_le2(g0 - 1, g1 - 1, r_lo, r_hi, u0, u1, u2, u3);
+      count_le2(g0 - 1, g1 - 1, 0, r_lo, r_hi, u0, u1, u2, u3);
       r_lo = r_lo < nb ? r_lo : nb;
       r_hi = r_hi < nb ? r_hi : nb;
       if (wg >= hs.Peff - 1) r_hi = nb;    // trailing row blocks without kept tiles
@@ -554,14 +584,31 @@ void fwd_kernel(const FwdParams prm) {
     // applies the same rule to both of its boundaries, so the ranges still tile the list.
     int r;
     {
+      // the row blocks in which the two ends of the range lie (positions behind a row block's tiles count as
+      // its end), then the tiles themselves
       int c0, c1, s0, e0, s1, e1;
-      count_le2(g0, g1, c0, c1, s0, e0, s1, e1);
+      count_le2(x0 + hs.lo, x1 + hs.lo, hs.gap, c0, c1, s0, e0, s1, e1);
       r = c0 - 1;
-      const int n0 = snap_boundary<C::SNAP>(g0, s0, e0);
+      g0 = tile_of_pos(hs, x0, r, s0, e0);
+      const int n0 = snap_boundary(snap, g0, s0, e0);
       if (n0 >= e0) ++r;
       g0 = n0;
-      if (g1 < hs.lo + hs.T) g1 = snap_boundary<C::SNAP>(g1, s1, e1);
+      if (x1 < hs.X) {
+        g1 = tile_of_pos(hs, x1, c1 - 1, s1, e1);
+        g1 = snap_boundary(snap, g1, s1, e1);
+      } else {
+        g1 = hs.lo + hs.T;
+      }
       if (g0 >= g1) return;
+    }
+    int kdone = -1, vdone = -1;
+    // The copies of this wavefront's first tile are asked for before anything else (its column index by one
+    // scalar load), so that they travel while the column list is staged and Q is read.
+    if (g0 + w < g1) {
+      const int c0 = flagged_col(g0 + w) & COL_MASK;
+      k_copy_all(kg + (int64_t)c0 * 64 * k_rs, g0 + w);
+      v_copy_all(vg + (int64_t)c0 * 64 * v_rs);
+      kdone = vdone = g0 + w;
     }
     stage_cols(g0, g1);
     if (threadIdx.x == 0) { ctr[0] = g0 + 2 * NW; ctr[3] = 0; }
@@ -569,7 +616,6 @@ void fwd_kernel(const FwdParams prm) {
     auto col_of = [&](int t) { return t - g0 < C::COLS_CAP ? lcols[t - g0] : flagged_col(t); };
     int cur = g0 + w, nxt = g0 + NW + w;      // the first two rounds are fixed
     int cb_nxt = nxt < g1 ? __builtin_amdgcn_readfirstlane(col_of(nxt)) : 0;   // column block of tile nxt
-    int kdone = -1, vdone = -1;
     int t = g0;
     const int32_t* rpg = prm.row_ptr + (int64_t)mh * nb;
     while (t < g1) {
@@ -641,6 +687,9 @@ void fwd_kernel(const FwdParams prm) {
       // groups of 4 registers (4 consecutive head-dimension values of one query per lane) over all
       // contributing wavefronts and writes them out.
       {
+        // (a wavefront without tiles in the range's first row block may still have its first tile's copies in
+        // flight: the merge borrows the tile buffers, so they are waited for and asked for again afterwards)
+        if (!mine) { wait_vm<0>(); kdone = -1; vdone = -1; }
         float lsum[2];
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) lsum[qb] = l_i[qb] + __shfl_xor(l_i[qb], 32);
@@ -746,9 +795,10 @@ void fwd_kernel(const FwdParams prm) {
           // The workgroups pf .. pl hold the parts of this row block: pf is the one before the first range
           // boundary that stays inside the row block (boundaries close to an end move there), pl the one
           // after the last.  Every holder computes the same two numbers.
-          int pl_ = split_of_tile(hs, row_e - 1), pf_ = split_of_tile(hs, row_s);
-          while (pl_ > pf_ && snap_boundary<C::SNAP>(split_begin(hs, pl_), row_s, row_e) >= row_e) --pl_;
-          while (pf_ < pl_ && snap_boundary<C::SNAP>(split_begin(hs, pf_ + 1), row_s, row_e) <= row_s) ++pf_;
+          const int64_t xrow = row_pos(hs, r, row_s);
+          int pl_ = split_of_pos(hs, xrow + (row_e - 1 - row_s)), pf_ = split_of_pos(hs, xrow);
+          while (pl_ > pf_ && snap_boundary(snap, tile_of_pos(hs, split_pos(hs, pl_), r, row_s, row_e), row_s, row_e) >= row_e) --pl_;
+          while (pf_ < pl_ && snap_boundary(snap, tile_of_pos(hs, split_pos(hs, pf_ + 1), r, row_s, row_e), row_s, row_e) <= row_s) ++pf_;
           const int nparts = pl_ - pf_ + 1;
           // The part is counted in once every wavefront's stores have been acknowledged (vmcnt 0, then the
           // barrier).  Every access to a part, stores here and loads below, is itself an access at device

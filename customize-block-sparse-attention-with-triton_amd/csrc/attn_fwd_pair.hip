@@ -199,6 +199,7 @@ __global__ __launch_bounds__(128, D == 128 ? 2 : 1) void fwd_pair_kernel(const F
   float m_i = 0.f, l_i = 0.f;
   uintx4 mfrag = {0u, 0u, 0u, 0u};
   bool fresh = true;
+  int any_m = 0;     // (wave-uniform) some lane's reference exponent is not zero: the extra contraction slice is needed
   __syncthreads();                                  // both halves of K(t0) and V(t0) are in LDS
 
   for (int t = t0; t < t1; ++t) {
@@ -230,8 +231,10 @@ __global__ __launch_bounds__(128, D == 128 ? 2 : 1) void fwd_pair_kernel(const F
       }
     }
     if constexpr (FOLD) {
-      s0 = mfma_qk<BF16>(ones_frag, mfrag, s0);
-      s1 = mfma_qk<BF16>(ones_frag, mfrag, s1);
+      if (any_m) {
+        s0 = mfma_qk<BF16>(ones_frag, mfrag, s0);
+        s1 = mfma_qk<BF16>(ones_frag, mfrag, s1);
+      }
     }
     if constexpr (EW) {
       if (partial) {
@@ -283,8 +286,11 @@ __global__ __launch_bounds__(128, D == 128 ? 2 : 1) void fwd_pair_kernel(const F
     };
     auto numerators = [&]() {
       float lnew = softmax_tile<FOLD, PB>(s0, s1, qk_scale, m_i, l_i, pf, 0);
-      if (__any(fresh || (EW && l_i == 0.f) || !(lnew - l_i < 16384.0f))) {
+      // (FOLD: the first tile of a row block keeps the reference at 0 when its sums are of moderate size)
+      const bool first = FOLD ? fresh && !(lnew >= 0.25f) : fresh;
+      if (__any(first || (EW && l_i == 0.f) || !(lnew - l_i < 16384.0f))) {
         recentre<DB, FOLD, EW>(s0, s1, oacc, 0, qk_scale, m_i, l_i, mfrag, fresh, g);
+        any_m = 1;
         lnew = softmax_tile<FOLD, PB>(s0, s1, qk_scale, m_i, l_i, pf, 0);
       }
       l_i = lnew;

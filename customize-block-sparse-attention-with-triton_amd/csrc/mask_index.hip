@@ -159,9 +159,15 @@ __device__ __forceinline__ int block_inclusive_sum(int v, int* s_w, int* total) 
   return v + before;
 }
 
+// FILL: the same workgroup also writes col_idx and groups, every thread the entries of its own segment (masks
+// of up to LISTS_FILL_MAX tiles, where one workgroup's scattered stores cost less than a second launch).
+constexpr int LISTS_FILL_MAX = 16384;
+template <bool FILL>
 __global__ __launch_bounds__(1024) void count_scan_kernel(const uint8_t* __restrict__ block, int rows, int nb,
                                                           int seg, int32_t* __restrict__ row_ptr,
-                                                          int32_t* __restrict__ gidx, int32_t* __restrict__ counts) {
+                                                          int32_t* __restrict__ gidx, int32_t* __restrict__ counts,
+                                                          int H, int32_t* __restrict__ col_idx,
+                                                          int32_t* __restrict__ groups) {
   constexpr int CH = LISTS_ONE_MAX_SEG / 16, WORDS = (CH + 1) / 2;
   __shared__ int s_w[16];
   __shared__ int s_off[1024];                   // kept tiles in front of a thread's segment
@@ -223,6 +229,24 @@ __global__ __launch_bounds__(1024) void count_scan_kernel(const uint8_t* __restr
   const int gi = block_inclusive_sum(len > 0 ? 1 : 0, s_w, &ngroups) - (len > 0 ? 1 : 0);
   if (tid < rows) gidx[tid] = gi;
   if (tid == 0) counts[0] = ngroups;
+  if constexpr (FILL) {
+    // entry number s_off[tid] + k of the list is the k-th set byte of this thread's segment: its column block
+    int pos = s_off[tid];
+#pragma unroll
+    for (int w = 0; w < WORDS; ++w) {
+      unsigned b = bits[w];
+      while (b != 0u) {
+        const int bit = __ffs(b) - 1;
+        b &= b - 1u;
+        col_idx[pos++] = (base + 32 * w + bit) % nb;
+      }
+    }
+    if (groups != nullptr && len > 0) {
+      const int bh = tid / nb;
+      int32_t* g = groups + (int64_t)gi * 5;
+      g[0] = bh / H; g[1] = bh % H; g[2] = tid % nb; g[3] = s_start[tid]; g[4] = len;
+    }
+  }
 }
 
 
@@ -482,7 +506,13 @@ int launch_block_mask_to_lists(const uint8_t* block, int Bm, int Hm, int nb, int
   const dim3 grid((rows + 3) / 4);
   if (contiguous && rows <= LISTS_ONE_MAX_ROWS && total <= 1024 * LISTS_ONE_MAX_SEG) {
     const int seg = (((int)total + 1023) / 1024 + 15) / 16 * 16;
-    hipLaunchKernelGGL(count_scan_kernel, dim3(1), dim3(1024), 0, st, block, rows, nb, seg, row_ptr, gidx, counts);
+    if (total <= LISTS_FILL_MAX) {      // (the whole call in one launch)
+      hipLaunchKernelGGL((count_scan_kernel<true>), dim3(1), dim3(1024), 0, st, block, rows, nb, seg, row_ptr, gidx, counts,
+                         Hm, col_idx, groups);
+      return launch_status();
+    }
+    hipLaunchKernelGGL((count_scan_kernel<false>), dim3(1), dim3(1024), 0, st, block, rows, nb, seg, row_ptr, gidx, counts,
+                       Hm, col_idx, groups);
   } else {
     hipLaunchKernelGGL(count_rows_kernel, grid, dim3(256), 0, st, block, rows, nb, Hm, sb, sh, sm, sn, cnt);
     hipLaunchKernelGGL(scan_rows_kernel, dim3(1), dim3(1024), 0, st, cnt, rows, row_ptr, gidx, counts);

@@ -32,6 +32,9 @@ _SIGNATURES = {
     "bsattn_fwd_workspace": ([_i, _i, _i, _i, ctypes.POINTER(ctypes.c_size_t)], _i),
     "bsattn_fwd": ([_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f,
                     _p, _p, _p, _p, _p, ctypes.c_size_t, _p], _i),
+    "bsattn_fwd_block_mask_workspace": ([_i, _i, _i, _i, _i, _i, ctypes.POINTER(ctypes.c_size_t)], _i),
+    "bsattn_fwd_block_mask": ([_p, _p, _p, _p, _p, _p, _p, _i, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f,
+                               _p, _p, _p, _p, _p, ctypes.c_size_t, _p], _i),
     "bsattn_fwd_static": ([_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f,
                            _p, _p, _p, _p, _p], _i),
     "bsattn_fwd_elementwise": ([_p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f,
@@ -86,8 +89,14 @@ def strides4(t):
     return _strides_array(t.stride())
 
 
+def raw_stream(device):
+    """The current stream of `device` as its raw handle (an int; 0 is the default stream)."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    return torch._C._cuda_getCurrentRawStream(index)
+
+
 def current_stream(device):
-    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    return ctypes.c_void_p(raw_stream(device))
 
 
 @functools.lru_cache(maxsize=256)
@@ -116,6 +125,22 @@ def _workspace_on(which, B, H, N, D, index):
         rc = fn(B, H, N, D, ctypes.byref(n))
     check(rc, which)
     return n.value
+
+
+@functools.lru_cache(maxsize=256)
+def _fused_workspace_on(Bm, Hm, B, H, N, D, index):
+    n = ctypes.c_size_t()
+    if index >= 0 and index != torch.cuda.current_device():
+        with torch.cuda.device(index):
+            rc = lib().bsattn_fwd_block_mask_workspace(Bm, Hm, B, H, N, D, ctypes.byref(n))
+    else:
+        rc = lib().bsattn_fwd_block_mask_workspace(Bm, Hm, B, H, N, D, ctypes.byref(n))
+    check(rc, "bsattn_fwd_block_mask_workspace")
+    return n.value
+
+
+def fwd_block_mask_workspace(Bm, Hm, B, H, N, D, device=None):
+    return _fused_workspace_on(Bm, Hm, B, H, N, D, _device_index(device))
 
 
 def fwd_workspace(B, H, N, D, device=None):

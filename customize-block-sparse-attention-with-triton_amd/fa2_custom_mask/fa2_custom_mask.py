@@ -10,7 +10,8 @@ import ctypes
 import torch
 
 from . import _ext
-from .utils import TILE, block_mask_to_lists, mask_to_lists, num_tiles, is_block_form, _check_mask
+from .utils import (TILE, TileLists, block_mask_to_lists, lists_cache, mask_to_lists, num_tiles, is_block_form,
+                    _check_mask)
 
 
 def build_groups_from_block_mask(mask):
@@ -29,6 +30,8 @@ def build_groups_from_block_mask(mask):
 
 def _prep(x):
     """Kernels need unit stride along the head dimension and 16-byte aligned rows."""
+    if x.is_contiguous() and (x.shape[3] * x.element_size()) % 16 == 0 and x.data_ptr() % 16 == 0:
+        return x                                                # (the usual case, decided without looking at strides)
     if x.stride(3) != 1 or any((s * x.element_size()) % 16 for s in x.stride()[:3]) or x.data_ptr() % 16:
         return x.contiguous()
     return x
@@ -51,11 +54,11 @@ def _workspace(nbytes, device):
     WORKSPACE_CACHE_BYTES is not kept), and nothing is kept or taken from it while a graph is being captured:
     memory first allocated under capture belongs to the graph's pool.  (Plans own their workspaces: they may be
     replayed from graphs on any stream.)"""
-    stream = torch.cuda.current_stream(device)
-    handle = ctypes.c_void_p(stream.cuda_stream)
+    raw = _ext.raw_stream(device)
+    handle = ctypes.c_void_p(raw)
     if torch.cuda.is_current_stream_capturing():
         return torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device), handle
-    key = (device.index, stream.cuda_stream)
+    key = (device.index, raw)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
@@ -73,6 +76,8 @@ def _like(x, dtype):
     101-103): the dimension order of x by stride, without gaps.  For q, k, v sliced out of one packed
     [B, N, 3, H, D] tensor that is [B, N, H, D] order behind a [B, H, N, D] shape."""
     t = torch.empty_like(x, dtype=dtype)
+    if x.is_contiguous() and x.shape[3] % 8 == 0:
+        return t
     if t.stride(3) != 1 or any((s * t.element_size()) % 16 for s in t.stride()[:3]):
         t = torch.empty(x.shape, dtype=dtype, device=x.device)
     return t
@@ -132,18 +137,34 @@ def set_deterministic(on):
     return bool(_ext.lib().bsattn_set_deterministic(1 if on else 0))
 
 
-def _forward(q, k, v, lists, sm_scale, out_dtype, want_lse):
-    B, H, N, D = q.shape
+def _plain(q, k, v):
+    """q, k, v of one shape without gaps and 16-byte aligned: one stride array serves all three and a result
+    laid out like them (the usual case, decided without looking at strides)."""
+    return (q.is_contiguous() and k.is_contiguous() and v.is_contiguous() and q.shape[3] % 8 == 0
+            and (q.data_ptr() | k.data_ptr() | v.data_ptr()) % 16 == 0)
+
+
+def _operands(q, k, v, out_dtype):
+    """(q, k, v, o, their four stride arrays) as the library takes them."""
+    if _plain(q, k, v):
+        o = torch.empty_like(q, dtype=out_dtype)                                # :59
+        sq = _ext.strides4(q)
+        return q, k, v, o, (sq, sq, sq, sq)
     q, k, v = _prep(q), _prep(k), _prep(v)
     o = _like(q, out_dtype)                                                     # :59
+    return q, k, v, o, (_ext.strides4(q), _ext.strides4(k), _ext.strides4(v), _ext.strides4(o))
+
+
+def _forward(q, k, v, lists, sm_scale, out_dtype, want_lse):
+    B, H, N, D = q.shape
+    q, k, v, o, strides = _operands(q, k, v, out_dtype)
     lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device) if want_lse else None  # :70
     wsb = _ext.fwd_workspace(B, H, N, D, q.device)
     ws, stream = _workspace(wsb, q.device)
     common = (lists.Bm, lists.Hm, B, H, N, D, _ext.dtype_code(q.dtype), _ext.dtype_code(out_dtype), float(sm_scale),
-              _ext.strides4(q), _ext.strides4(k), _ext.strides4(v), _ext.strides4(o),
-              ws.data_ptr(), wsb, stream)
+              *strides, ws.data_ptr(), wsb, stream)
     ptrs = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr() if want_lse else None,
-            lists.row_ptr.data_ptr(), lists.col_idx.data_ptr())
+            lists.row_ptr_ptr, lists.col_idx_ptr)
     if lists.bits is None:
         rc = _ext.lib().bsattn_fwd(*ptrs, *common)
     else:                                      # elementwise mask: exact inside partly set tiles
@@ -171,10 +192,10 @@ class ForwardPlan:
         tail = (lists.Bm, lists.Hm, B, H, N, D, _ext.dtype_code(q.dtype), _ext.dtype_code(out_dtype),
                 float(sm_scale)) + self._keep + (self.ws.data_ptr(), wsb, ctypes.c_void_p(stream.cuda_stream))
         head = (self.q.data_ptr(), self.k.data_ptr(), self.v.data_ptr(), self.o.data_ptr(), self.lse.data_ptr(),
-                lists.row_ptr.data_ptr())
+                lists.row_ptr_ptr)
         if lists.bits is not None:
             raise ValueError("a plan takes block masks only")
-        self._args = head + (lists.col_idx.data_ptr(),) + tail
+        self._args = head + (lists.col_idx_ptr,) + tail
         self._fn = _ext.lib().bsattn_fwd
 
     def run(self):
@@ -192,8 +213,8 @@ def _backward(q, k, v, o, do, lse, lists, lists_t, sm_scale, out_dtype):
     ws, stream = _workspace(wsb, q.device)
     tensors = (q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), do.data_ptr(), lse.data_ptr(),
                dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
-               lists.row_ptr.data_ptr(), lists.col_idx.data_ptr(), lists_t.row_ptr.data_ptr(),
-               lists_t.col_idx.data_ptr())
+               lists.row_ptr_ptr, lists.col_idx_ptr, lists_t.row_ptr_ptr,
+               lists_t.col_idx_ptr)
     common = (lists.Bm, lists.Hm, B, H, N, D,
               _ext.dtype_code(q.dtype), _ext.dtype_code(out_dtype), float(sm_scale),
               _ext.strides4(q), _ext.strides4(k), _ext.strides4(v), _ext.strides4(o), _ext.strides4(do),
@@ -226,8 +247,8 @@ class BackwardPlan:
         stream = stream if stream is not None else torch.cuda.current_stream(q.device)
         self._args = (self.q.data_ptr(), self.k.data_ptr(), self.v.data_ptr(), self.o.data_ptr(), self.do.data_ptr(),
                       lse.data_ptr(), self.dq.data_ptr(), self.dk.data_ptr(), self.dv.data_ptr(),
-                      lists.row_ptr.data_ptr(), lists.col_idx.data_ptr(), lists_t.row_ptr.data_ptr(),
-                      lists_t.col_idx.data_ptr(), lists.Bm, lists.Hm, B, H, N, D, _ext.dtype_code(q.dtype),
+                      lists.row_ptr_ptr, lists.col_idx_ptr, lists_t.row_ptr_ptr,
+                      lists_t.col_idx_ptr, lists.Bm, lists.Hm, B, H, N, D, _ext.dtype_code(q.dtype),
                       _ext.dtype_code(out_dtype), float(sm_scale)) + self._keep + (
                           self.ws.data_ptr(), wsb, ctypes.c_void_p(stream.cuda_stream))
         self._fn = _ext.lib().bsattn_bwd
@@ -239,16 +260,47 @@ class BackwardPlan:
         return self.dq, self.dk, self.dv
 
 
+def _forward_from_block_mask(q, k, v, mask, sm_scale, out_dtype, want_lse):
+    """Lists and forward from one call into the library (bsattn_fwd_block_mask), for a block mask whose lists
+    are not in the cache: one buffer for the lists, one for the result, and the stream's workspace."""
+    B, H, N, D = q.shape
+    Bm, Hm, nb = mask.shape[0], mask.shape[1], mask.shape[2]
+    q, k, v, o, strides = _operands(q, k, v, out_dtype)
+    lists = TileLists(Bm, Hm, nb, q.device)
+    lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device) if want_lse else None
+    wsb = _ext.fwd_block_mask_workspace(Bm, Hm, B, H, N, D, q.device)
+    ws, stream = _workspace(wsb, q.device)
+    rc = _ext.lib().bsattn_fwd_block_mask(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr() if want_lse else None,
+        mask.data_ptr(), _ext.strides4(mask), Bm, Hm, lists.row_ptr_ptr, lists.col_idx_ptr, lists.counts_ptr,
+        B, H, N, D, _ext.dtype_code(q.dtype), _ext.dtype_code(out_dtype), float(sm_scale),
+        *strides, ws.data_ptr(), wsb, stream)
+    _ext.check(rc, "bsattn_fwd_block_mask")
+    return o, lse, lists
+
+
 def _forward_only(q, k, v, mask, sm_scale, out_fp32, return_lse):
     """The forward of _attention without anything kept for a backward."""
     B, H, N, D = _check_qkv(q, k, v, mask)
     if mask is None:
         mask = _dense_mask(q.device, num_tiles(N))
-    lists = mask_to_lists(mask, N)
+    out_dtype = torch.float32 if out_fp32 else q.dtype
+    whole = N % TILE == 0 and D >= 64
+    lists = lists_cache.get(mask, N, False)
+    if lists is None and whole and mask.shape[2] * TILE == N:
+        # a block mask seen for the first time (or one that changes with every call): lists and forward in one call
+        o, lse, lists = _forward_from_block_mask(q, k, v, mask, sm_scale, out_dtype, return_lse)
+        lists_cache.put(mask, N, False, lists)
+        return (o, lse) if return_lse else o
+    if lists is None:
+        lists = mask_to_lists(mask, N)
+    if whole:
+        o, lse = _forward(q, k, v, lists, sm_scale, out_dtype, return_lse)
+        return (o, lse) if return_lse else o
     q, k, v = _padded(q, N, D), _padded(k, N, D), _padded(v, N, D)
-    o, lse = _forward(q, k, v, lists, sm_scale, torch.float32 if out_fp32 else q.dtype, True)
+    o, lse = _forward(q, k, v, lists, sm_scale, out_dtype, return_lse)
     if o.shape[2:] != (N, D):
-        o, lse = o[:, :, :N, :D], lse[:, :, :N]
+        o, lse = o[:, :, :N, :D], (lse[:, :, :N] if lse is not None else None)
     return (o, lse) if return_lse else o
 
 

@@ -27,15 +27,55 @@ class TileLists:
     """Device-resident kept-tile lists of a block mask [Bm, Hm, nb, nb] (fixed shapes, no
     host synchronisation): row_ptr int32 [Bm*Hm*nb+1], col_idx int32 [Bm*Hm*nb*nb] (first T
     entries valid), counts int32 [2] = (G, T), groups int32 [Bm*Hm*nb, 5] (first G rows
-    valid) or None."""
+    valid) or None.  All of them live in one int32 buffer (workspace | row_ptr | counts | col_idx | groups);
+    the tensor views are made when first asked for, the calls into the library only need the addresses."""
 
-    __slots__ = ("row_ptr", "col_idx", "groups", "counts", "Bm", "Hm", "nb", "partial", "bits")
+    __slots__ = ("buf", "Bm", "Hm", "nb", "has_groups", "partial", "bits", "_views",
+                 "ws_ptr", "ws_bytes", "row_ptr_ptr", "counts_ptr", "col_idx_ptr", "groups_ptr", "_off")
 
-    def __init__(self, row_ptr, col_idx, groups, counts, Bm, Hm, nb):
-        self.row_ptr, self.col_idx, self.groups, self.counts = row_ptr, col_idx, groups, counts
-        self.Bm, self.Hm, self.nb = Bm, Hm, nb
+    def __init__(self, Bm, Hm, nb, device, want_groups=False):
+        rows = Bm * Hm * nb
+        wsb = _ext.mask_lists_workspace(Bm, Hm, nb)
+        o_ptr = (wsb + 3) // 4
+        o_counts = o_ptr + rows + 1
+        o_cols = o_counts + 2
+        o_groups = o_cols + rows * nb
+        self.buf = torch.empty(o_groups + (rows * 5 if want_groups else 0), dtype=torch.int32, device=device)
+        self.Bm, self.Hm, self.nb, self.has_groups = Bm, Hm, nb, want_groups
+        self._off = (o_ptr, o_counts, o_cols, o_groups)
+        base = self.buf.data_ptr()
+        self.ws_ptr, self.ws_bytes = base, wsb
+        self.row_ptr_ptr, self.counts_ptr = base + 4 * o_ptr, base + 4 * o_counts
+        self.col_idx_ptr = base + 4 * o_cols
+        self.groups_ptr = base + 4 * o_groups if want_groups else None
         # elementwise masks only: per kept tile "partly set" flag and packed 64 x 64 bits
         self.partial, self.bits = None, None
+        self._views = None
+
+    def _make_views(self):
+        if self._views is None:
+            o_ptr, o_counts, o_cols, o_groups = self._off
+            b = self.buf
+            rows = self.Bm * self.Hm * self.nb
+            self._views = (b[o_ptr:o_counts], b[o_counts:o_cols], b[o_cols:o_groups],
+                           b[o_groups:].view(rows, 5) if self.has_groups else None)
+        return self._views
+
+    @property
+    def row_ptr(self):
+        return self._make_views()[0]
+
+    @property
+    def counts(self):
+        return self._make_views()[1]
+
+    @property
+    def col_idx(self):
+        return self._make_views()[2]
+
+    @property
+    def groups(self):
+        return self._make_views()[3]
 
 
 def _check_mask(mask):
@@ -72,28 +112,15 @@ def block_mask_to_lists(block, transpose=False, want_groups=False):
     Bm, Hm, nb, nb2 = block.shape
     if nb != nb2:
         raise ValueError("block mask must be square")
-    dev = block.device
-    rows = Bm * Hm * nb
-    # one allocation for everything the call writes: workspace | row_ptr | counts | col_idx | groups
-    wsb = _ext.mask_lists_workspace(Bm, Hm, nb)
-    ws_ints = (wsb + 3) // 4
-    o_ptr = ws_ints
-    o_counts = o_ptr + rows + 1
-    o_cols = o_counts + 2
-    o_groups = o_cols + rows * nb
-    buf = torch.empty(o_groups + (rows * 5 if want_groups else 0), dtype=torch.int32, device=dev)
-    ws = buf[:ws_ints]
-    row_ptr, counts, col_idx = buf[o_ptr:o_counts], buf[o_counts:o_cols], buf[o_cols:o_groups]
-    groups = buf[o_groups:].view(rows, 5) if want_groups else None
+    lists = TileLists(Bm, Hm, nb, block.device, want_groups)
     sb, sh, sm, sn = block.stride()
     if transpose:
         sm, sn = sn, sm
     rc = _ext.lib().bsattn_block_mask_to_lists(
-        block.data_ptr(), Bm, Hm, nb, sb, sh, sm, sn, row_ptr.data_ptr(), col_idx.data_ptr(),
-        groups.data_ptr() if want_groups else None, counts.data_ptr(), ws.data_ptr(), wsb,
-        _ext.current_stream(dev))
+        block.data_ptr(), Bm, Hm, nb, sb, sh, sm, sn, lists.row_ptr_ptr, lists.col_idx_ptr,
+        lists.groups_ptr, lists.counts_ptr, lists.ws_ptr, lists.ws_bytes, _ext.current_stream(block.device))
     _ext.check(rc, "bsattn_block_mask_to_lists")
-    return TileLists(row_ptr, col_idx, groups, counts, Bm, Hm, nb)
+    return lists
 
 
 def pack_mask_tiles(mask, lists, transpose=False):
@@ -114,8 +141,8 @@ def pack_mask_tiles(mask, lists, transpose=False):
     cap = Bm * Hm * lists.nb * lists.nb
     partial = torch.empty(cap, dtype=torch.uint8, device=mask.device)
     bits = torch.empty((cap, 64), dtype=torch.int64, device=mask.device)
-    rc = _ext.lib().bsattn_pack_mask_tiles(mask.data_ptr(), Bm, Hm, N, sb, sh, sm, sn, lists.row_ptr.data_ptr(),
-                                           lists.col_idx.data_ptr(), partial.data_ptr(), bits.data_ptr(),
+    rc = _ext.lib().bsattn_pack_mask_tiles(mask.data_ptr(), Bm, Hm, N, sb, sh, sm, sn, lists.row_ptr_ptr,
+                                           lists.col_idx_ptr, partial.data_ptr(), bits.data_ptr(),
                                            _ext.current_stream(mask.device))
     _ext.check(rc, "bsattn_pack_mask_tiles")
     return partial, bits
@@ -153,7 +180,7 @@ def gather_mask_tiles(grid_partial, grid_bits, lists, transpose=False):
     partial = torch.empty(cap, dtype=torch.uint8, device=dev)
     bits = torch.empty((cap, 64), dtype=torch.int64, device=dev)
     rc = _ext.lib().bsattn_gather_mask_tiles(grid_partial.data_ptr(), grid_bits.data_ptr(), lists.Bm, lists.Hm, lists.nb,
-                                             1 if transpose else 0, lists.row_ptr.data_ptr(), lists.col_idx.data_ptr(),
+                                             1 if transpose else 0, lists.row_ptr_ptr, lists.col_idx_ptr,
                                              partial.data_ptr(), bits.data_ptr(), _ext.current_stream(dev))
     _ext.check(rc, "bsattn_gather_mask_tiles")
     return partial, bits
@@ -168,7 +195,7 @@ def tail_mask_tiles(lists, valid_last, transpose=False):
     partial = torch.empty(cap, dtype=torch.uint8, device=dev)
     bits = torch.empty((cap, 64), dtype=torch.int64, device=dev)
     rc = _ext.lib().bsattn_tail_mask_tiles(lists.Bm, lists.Hm, lists.nb, valid_last, 1 if transpose else 0,
-                                           lists.row_ptr.data_ptr(), lists.col_idx.data_ptr(), partial.data_ptr(),
+                                           lists.row_ptr_ptr, lists.col_idx_ptr, partial.data_ptr(),
                                            bits.data_ptr(), _ext.current_stream(dev))
     _ext.check(rc, "bsattn_tail_mask_tiles")
     return partial, bits
@@ -205,7 +232,7 @@ class _ListsCache:
 
     def __init__(self, capacity=8):
         self.capacity = capacity
-        # (weakref to mask, version, N, transpose, lists, stream the lists were built on, event), most recent last
+        # (weakref to mask, version, N, transpose, lists, stream the lists were built on), most recent last
         self._entries = []
 
     @staticmethod
@@ -221,13 +248,16 @@ class _ListsCache:
         version = self._version(mask)
         if version is None:
             return None
-        for i, (ref, ver, n, tr, lists, stream, ready) in enumerate(self._entries):
+        for i, (ref, ver, n, tr, lists, stream) in enumerate(self._entries):
             if ref() is mask and ver == version and n == N and tr == transpose:
-                self._entries.append(self._entries.pop(i))
-                # the lists were filled by kernels on `stream`: work on another stream waits for them
-                current = torch.cuda.current_stream(mask.device)
-                if current != stream:
-                    current.wait_event(ready)
+                if i != len(self._entries) - 1:
+                    self._entries.append(self._entries.pop(i))
+                # the lists were filled by kernels on `stream` (a raw handle): work on another stream waits for
+                # what that stream has been given so far (no event is recorded when the lists are made: a mask
+                # that changes with every call would pay for it every time)
+                if _ext.raw_stream(mask.device) != stream:
+                    torch.cuda.current_stream(mask.device).wait_stream(
+                        torch.cuda.ExternalStream(stream, device=mask.device) if stream else torch.cuda.default_stream(mask.device))
                 return lists
         return None
 
@@ -235,12 +265,9 @@ class _ListsCache:
         version = self._version(mask)
         if version is None:
             return
-        stream = torch.cuda.current_stream(mask.device)
-        ready = torch.cuda.Event()
-        ready.record(stream)
-        self._entries = [e for e in self._entries if e[0]() is not None]
-        self._entries.append((weakref.ref(mask), version, N, transpose, lists, stream, ready))
-        del self._entries[:-self.capacity]
+        if len(self._entries) >= self.capacity:
+            self._entries = [e for e in self._entries if e[0]() is not None][-(self.capacity - 1):]
+        self._entries.append((weakref.ref(mask), version, N, transpose, lists, _ext.raw_stream(mask.device)))
 
     def clear(self):
         self._entries = []

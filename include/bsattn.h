@@ -191,6 +191,23 @@ int bsattn_fwd(const void* q, const void* k, const void* v, void* o, float* lse,
                const int64_t* o_strides, void* workspace, size_t workspace_bytes,
                void* stream);
 
+/* The reference's whole forward call in one: _attention.forward (fa2_custom_mask/fa2_custom_mask.py:43-94) builds
+ * the lists of the block mask (:48) and launches _attn_fwd on them (:77-87).  This entry point enqueues
+ * bsattn_block_mask_to_lists (without `groups`) and bsattn_fwd on `stream` from one host call, for callers
+ * whose mask changes from call to call; row_ptr, col_idx (capacities as for bsattn_block_mask_to_lists) and
+ * counts are left filled and may be handed to later bsattn_fwd / bsattn_bwd calls for the same mask.
+ * mask_strides: the four element strides of the bool [Bm,Hm,nb,nb] mask, nb = N / 64 (0 or any value for
+ * dimensions of size 1).  One workspace of bsattn_fwd_block_mask_workspace bytes (16-byte aligned) serves both
+ * steps.  All arguments are checked before the first launch. */
+int bsattn_fwd_block_mask_workspace(int Bm, int Hm, int B, int H, int N, int D, size_t* bytes);
+int bsattn_fwd_block_mask(const void* q, const void* k, const void* v, void* o, float* lse,
+                          const uint8_t* block, const int64_t* mask_strides, int Bm, int Hm,
+                          int32_t* row_ptr, int32_t* col_idx, int32_t* counts,
+                          int B, int H, int N, int D, int dtype, int out_dtype, float sm_scale,
+                          const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                          const int64_t* o_strides, void* workspace, size_t workspace_bytes,
+                          void* stream);
+
 /* Forward that allocates nothing and needs no workspace argument.  It has no counterpart in the
  * reference; it is for callers that cannot allocate device memory around the call: code under HIP
  * graph capture, tight serving loops, harnesses that forbid allocation.  Same arguments, results and

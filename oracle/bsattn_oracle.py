@@ -230,7 +230,7 @@ def tiled_attention(q, k, v, groups, n_list, sm_scale, dtype=np.float32, p_round
 # ----------------------------------------------------------------------------
 # backward: the gradient algebra the reference intends
 # ----------------------------------------------------------------------------
-def attention_backward(q, k, v, block_mask, sm_scale, do, dtype=np.float32):
+def attention_backward(q, k, v, block_mask, sm_scale, do, dtype=np.float32, o_stored=None):
     """Gradient of naive_attention w.r.t. q,k,v for upstream gradient `do`.
 
     Algebra of fa2_custom_mask/fa2_bwd.py: delta = rowsum(O*dO) (:17); P = softmax
@@ -239,6 +239,10 @@ def attention_backward(q, k, v, block_mask, sm_scale, do, dtype=np.float32):
     dQ = dS K * sm_scale (:130 with the host pre-scale fa2_custom_mask.py:110-111, :284).
     Evaluated over full rows (all kept tiles), which is what a correct block-sparse
     backward must equal.  Returns (dq, dk, dv, delta).
+
+    o_stored: the forward's output as it was stored (fp16 / bf16 values).  The reference takes delta from that
+    tensor (fa2_custom_mask.py:114-121 hands the saved `o` to _attn_bwd_preprocess, fa2_bwd.py:15-17), not from
+    an exact O; the difference only shows where delta is large against dP - delta.  None: the exact O.
     """
     q = np.asarray(q, dtype=dtype); k = np.asarray(k, dtype=dtype); v = np.asarray(v, dtype=dtype)
     do = np.asarray(do, dtype=dtype)
@@ -256,7 +260,7 @@ def attention_backward(q, k, v, block_mask, sm_scale, do, dtype=np.float32):
             p = np.exp(s - mx)
             den = p.sum(axis=1, keepdims=True)
             p = p / np.where(den > 0, den, dtype(1))
-            o = p @ v[b, h]
+            o = p @ v[b, h] if o_stored is None else np.asarray(o_stored, dtype=dtype)[b, h]
             dl = (o * do[b, h]).sum(axis=1)                        # fa2_bwd.py:17
             dv[b, h] = p.T @ do[b, h]                              # :67
             dp = do[b, h] @ v[b, h].T                              # :71

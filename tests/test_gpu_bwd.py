@@ -212,27 +212,32 @@ def test_large_magnitudes_backward_d128_fp16(dev):
     (so lse / sm_scale does too) and delta = rowsum(O dO) above 1e5 (values with a large common component, as
     gradients under loss scaling meet them), while P and dS = P (dP - delta) themselves stay representable (the
     reference rounds both to fp16 as well, fa2_bwd.py:66,73,127).  The dK/dV kernel feeds lse and delta through a
-    contraction slice as 16-bit pieces: they must not overflow."""
+    contraction slice as 16-bit pieces: they must not overflow.  With delta this large against dP - delta the
+    rounding of the stored O matters (1 % of dQ and dK here): the oracle takes delta from the same fp16 O the
+    kernels are given, as the reference does (fa2_bwd.py:15-17)."""
     import fa2_custom_mask as fm
     B, H, N, D = 1, 2, 512, 128
     g = torch.Generator().manual_seed(91)
     q = (torch.randn(B, H, N, D, generator=g) * 40.0).to(torch.float16)
     k = (torch.randn(B, H, N, D, generator=g) * 40.0).to(torch.float16)
     v0 = 300.0 * torch.sign(torch.randn(1, H, 1, D, generator=g))
-    v = (v0 + torch.randn(B, H, N, D, generator=g)).to(torch.float16)
+    v = (v0 + 20.0 * torch.randn(B, H, N, D, generator=g)).to(torch.float16)
     do = (torch.randn(B, H, N, D, generator=g) * 30.0).to(torch.float16)
     mask = uniform_block_mask(1, 1, 8, 0.5, 13)
     sc = 0.001
     o_r, lse_r = orc.naive_attention(f32(q), f32(k), f32(v), mask.numpy(), sc, return_lse=True)
-    dq_r, dk_r, dv_r, delta_r = orc.attention_backward(f32(q), f32(k), f32(v), mask.numpy(), sc, f32(do))
-    assert np.abs(delta_r).max() > 65504.0 and np.abs(lse_r).max() / sc > 65504.0     # the case this test is for
     o, lse, dq, dk, dv = fm.attention_forward_backward(q.to(dev), k.to(dev), v.to(dev), mask.to(dev), sc, do.to(dev),
                                                        out_fp32=True)
     torch.cuda.synchronize()
+    assert errors(o, o_r)[1] <= 2e-3
+    o16 = o.to(torch.float16)                   # what attention_forward_backward hands to the backward
+    dq_r, dk_r, dv_r, delta_r = orc.attention_backward(f32(q), f32(k), f32(v), mask.numpy(), sc, f32(do),
+                                                       dtype=np.float64, o_stored=f32(o16))
+    assert np.abs(delta_r).max() > 65504.0 and np.abs(lse_r).max() / sc > 65504.0     # the case this test is for
     for name, got, ref in (("dQ", dq, dq_r), ("dK", dk, dk_r), ("dV", dv, dv_r)):
         assert bool(torch.isfinite(got).all()), name
         ma, rl = errors(got, ref)
         print("%s: max-abs %.3e of %.3e, rel-L2 %.3e" % (name, ma, float(np.abs(ref).max()), rl))
         # (the softmax is nearly one-hot and the exponents carry the rounding of the 16-bit scaled Q: a looser
         # bar than for N(0,1) data; an overflowing piece gives NaN or errors of the size of the result)
-        assert rl <= 1e-2, name
+        assert rl <= 5e-3, name

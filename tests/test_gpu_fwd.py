@@ -329,3 +329,56 @@ def test_large_magnitudes(dev, dtype, out_fp32):
     assert ma <= (2e-2 if dtype == torch.float16 else 3e-2) * max(1.0, scale / 4.0)
     assert rl <= (1e-3 if dtype == torch.float16 or out_fp32 else 3e-3) * 1.5
     assert np.abs(lse.cpu().numpy() - lse_ref).max() <= 2e-3 * max(1.0, float(np.abs(lse_ref).max()) / 8.0)
+
+
+@pytest.mark.parametrize("B,H,Bm,Hm,N,D,dtype", [(1, 1, 1, 1, 1024, 64, torch.float16), (2, 3, 1, 1, 512, 128, torch.bfloat16),
+                                                 (2, 2, 2, 2, 768, 64, torch.float16), (1, 2, 1, 2, 4096, 64, torch.float16)])
+def test_lists_and_forward_from_one_call(dev, B, H, Bm, Hm, N, D, dtype):
+    """bsattn_fwd_block_mask (the reference's whole forward call, fa2_custom_mask.py:43-94: lists of the block mask,
+    then the kernel): O and LSE against the oracle, the lists it leaves against the oracle's, bit for bit, and the
+    same through flash_attention_custom_mask for a mask that is not in the cache."""
+    import ctypes
+    import fa2_custom_mask as fm
+    from fa2_custom_mask import _ext, utils
+    nb = N // 64
+    mask = uniform_block_mask(Bm, Hm, nb, 0.4, 300 + N)
+    mask[0, 0, 1, :] = False                      # a row block without kept tiles
+    q, k, v = make_qkv(B, H, N, D, dtype, 301 + N)
+    sc = 1.0 / np.sqrt(D)
+    o_ref, lse_ref = orc.naive_attention(f32(q), f32(k), f32(v), mask.numpy(), sc, return_lse=True)
+    qd, kd, vd, md = q.to(dev), k.to(dev), v.to(dev), mask.to(dev)
+    lib = _ext.lib()
+    rows = Bm * Hm * nb
+    row_ptr = torch.full((rows + 1,), -1, dtype=torch.int32, device=dev)
+    col_idx = torch.full((rows * nb,), -1, dtype=torch.int32, device=dev)
+    counts = torch.full((2,), -1, dtype=torch.int32, device=dev)
+    o = torch.full((B, H, N, D), float("nan"), dtype=dtype, device=dev)
+    lse = torch.full((B, H, N), float("nan"), dtype=torch.float32, device=dev)
+    n = ctypes.c_size_t()
+    assert lib.bsattn_fwd_block_mask_workspace(Bm, Hm, B, H, N, D, ctypes.byref(n)) == 0
+    ws = torch.randint(0, 255, (n.value,), dtype=torch.uint8, device=dev)       # contents must not matter
+    args = (qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o.data_ptr(), lse.data_ptr(), md.data_ptr(), _ext.strides4(md),
+            Bm, Hm, row_ptr.data_ptr(), col_idx.data_ptr(), counts.data_ptr(), B, H, N, D, _ext.dtype_code(dtype),
+            _ext.dtype_code(dtype), float(sc), _ext.strides4(qd), _ext.strides4(kd), _ext.strides4(vd), _ext.strides4(o))
+    assert lib.bsattn_fwd_block_mask(*args, ws.data_ptr(), n.value - 1, _ext.current_stream(dev)) == -6   # workspace too small
+    assert lib.bsattn_fwd_block_mask(*args, ws.data_ptr(), n.value, _ext.current_stream(dev)) == 0
+    torch.cuda.synchronize()
+    rp_ref, ci_ref = orc.csr_from_block_mask(mask.numpy())
+    G, T = counts.tolist()
+    assert T == len(ci_ref) and G == int((np.diff(rp_ref) > 0).sum())
+    assert np.array_equal(row_ptr.cpu().numpy(), rp_ref) and np.array_equal(col_idx[:T].cpu().numpy(), ci_ref)
+    tol_abs, tol_rel = (2e-2, 1e-3) if dtype == torch.float16 else (3e-2, 3e-3)
+    ma, rl = errors(o, o_ref)
+    assert ma <= tol_abs and rl <= tol_rel
+    fin = np.isfinite(lse_ref)
+    assert np.abs(lse.cpu().numpy()[fin] - lse_ref[fin]).max() <= 2e-3 and bool(torch.isinf(lse[0, 0, 64:128]).all())
+    # the Python operator takes the same route for a mask it has not seen
+    utils.lists_cache.clear()
+    o2 = fm.flash_attention_custom_mask(qd, kd, vd, md, sc)
+    cached = utils.lists_cache.get(md, N, False)
+    assert cached is not None and np.array_equal(cached.row_ptr.cpu().numpy(), rp_ref)
+    ma, rl = errors(o2, o_ref)
+    assert ma <= tol_abs and rl <= tol_rel
+    o3, lse3 = fm.flash_attention_custom_mask_lse(qd, kd, vd, md, sc)            # second call: cached lists
+    assert same_up_to_rounding(o3, o2, rel=2.0 ** -9 if dtype == torch.float16 else 2.0 ** -6, abs_=3e-4 if dtype == torch.float16 else 2e-3)
+    assert np.abs(lse3.cpu().numpy()[fin] - lse_ref[fin]).max() <= 2e-3

@@ -30,7 +30,12 @@ def _check_lists(mask_cpu, dev):
                                         # (1023 rows, 256 KB of block mask)
                                         ((1, 1, 512, 512), 0.5), ((1, 1, 513, 513), 0.5), ((1, 1023, 1, 1), 0.5),
                                         ((1, 1024, 1, 1), 0.5), ((1, 31, 33, 33), 0.3), ((1, 32, 32, 32), 0.3),
-                                        ((1, 1, 512, 512), 1.0), ((2, 2, 255, 255), 0.02)])
+                                        ((1, 1, 512, 512), 1.0), ((2, 2, 255, 255), 0.02),
+                                        # either side of the size up to which the same workgroup also fills the
+                                        # lists (16384 tiles): full, sparse, several heads, an odd row length
+                                        ((1, 1, 128, 128), 1.0), ((1, 1, 128, 128), 0.03), ((1, 1, 129, 129), 0.5),
+                                        ((2, 2, 64, 64), 0.5), ((1, 4, 64, 64), 1.0), ((1, 3, 73, 73), 0.2),
+                                        ((1, 1, 127, 127), 0.97), ((1, 7, 5, 5), 0.5)])
 def test_groups_random(dev, shape, keep):
     g = torch.Generator().manual_seed(7)
     _check_lists(torch.rand(*shape, generator=g) < keep, dev)

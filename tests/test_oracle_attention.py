@@ -127,6 +127,29 @@ def test_backward_equals_autograd(seed):
     assert np.abs(delta - (out * do).sum(-1)).max() < 1e-11                   # fa2_bwd.py:17
 
 
+def test_backward_with_stored_output():
+    """o_stored only replaces the O that delta is taken from.  Given the exact O the gradients are the autograd
+    ones; given O + E the change is what the algebra fixes: delta' = delta + rowsum(E dO), dV unchanged,
+    dQ' - dQ = -(P * rowsum(E dO)) K sm_scale and dK' - dK = -(P * rowsum(E dO))^T Q sm_scale, with P taken from
+    torch's own softmax."""
+    q, k, v, mask, sc = rand_case(5, B=1, H=2, nb=3, D=64)
+    rng = np.random.default_rng(55)
+    do = rng.standard_normal(q.shape)
+    (dq_r, dk_r, dv_r), out = torch_grads(q, k, v, mask, sc, do)
+    dq, dk, dv, delta = orc.attention_backward(q, k, v, mask, sc, do, dtype=np.float64, o_stored=out)
+    for a, b in ((dq, dq_r), (dk, dk_r), (dv, dv_r)):
+        assert np.abs(a - b).max() < 1e-11
+    E = 0.01 * rng.standard_normal(q.shape)
+    dq2, dk2, dv2, delta2 = orc.attention_backward(q, k, v, mask, sc, do, dtype=np.float64, o_stored=out + E)
+    shift = (E * do).sum(-1)
+    assert np.abs(delta2 - delta - shift).max() < 1e-11 and np.abs(dv2 - dv).max() == 0.0
+    em = torch.tensor(mask).repeat_interleave(64, 2).repeat_interleave(64, 3)
+    sm = torch.softmax((torch.tensor(q) @ torch.tensor(k).transpose(-1, -2) * sc).masked_fill(~em, float("-inf")), -1)
+    corr = sm * torch.tensor(shift)[..., None]
+    assert np.abs((dq2 - dq) + (corr @ torch.tensor(k)).numpy() * sc).max() < 1e-11
+    assert np.abs((dk2 - dk) + (corr.transpose(-1, -2) @ torch.tensor(q)).numpy() * sc).max() < 1e-11
+
+
 def test_backward_finite_differences():
     rng = np.random.default_rng(9)
     q, k, v, mask, sc = rand_case(9, B=1, H=1, nb=2, D=16)
