@@ -191,6 +191,21 @@ __global__ __launch_bounds__(128, D == 256 ? 1 : 2) void dq_kernel(const BwdPara
   const int mh = (prm.Bm > 1 ? b : 0) * prm.Hm + (prm.Hm > 1 ? h : 0);
   const cint_ptr_t rp = (cint_ptr_t)(uintptr_t)(prm.row_ptr + (int64_t)mh * nb);
   const cint_ptr_t cols = (cint_ptr_t)(uintptr_t)prm.col_idx;
+  // The rows this workgroup owns for its whole walk (Q, dO, O, lse of its queries) depend on the block index only:
+  // they are asked for first, and travel while the list is looked up and the first tiles are requested.
+  const int64_t qrow = (int64_t)m * 64 + 32 * wv + ln;
+  const unsigned short* qp = (const unsigned short*)prm.q + b * prm.qs[0] + h * prm.qs[1] + qrow * prm.qs[2];
+  const unsigned short* gp = (const unsigned short*)prm.d_o + b * prm.dos[0] + h * prm.dos[1] + qrow * prm.dos[2];
+  const unsigned short* op = (const unsigned short*)prm.o + b * prm.os[0] + h * prm.os[1] + qrow * prm.os[2];
+  uintx4 qfr[KS], dofr[KS], ofr[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    qfr[s] = *reinterpret_cast<const uintx4*>(qp + 16 * s + 8 * g);
+    dofr[s] = *reinterpret_cast<const uintx4*>(gp + 16 * s + 8 * g);
+  }
+#pragma unroll
+  for (int s = 0; s < KS; ++s) ofr[s] = *reinterpret_cast<const uintx4*>(op + 16 * s + 8 * g);
+  const float lse_q = prm.lse[(int64_t)bh * prm.N + qrow];
   int u0, u1;                                                  // steps: tile u / STEPS, part u % STEPS
   {
     const int t0 = rp[m], len = rp[m + 1] - t0;                // this workgroup's share of the row's list
@@ -213,26 +228,15 @@ __global__ __launch_bounds__(128, D == 256 ? 1 : 2) void dq_kernel(const BwdPara
   };
   if (u0 < u1) issue(u0, 0);
 
-  const int64_t qrow = (int64_t)m * 64 + 32 * wv + ln;
-  const unsigned short* qp = (const unsigned short*)prm.q + b * prm.qs[0] + h * prm.qs[1] + qrow * prm.qs[2];
-  const unsigned short* gp = (const unsigned short*)prm.d_o + b * prm.dos[0] + h * prm.dos[1] + qrow * prm.dos[2];
-  uintx4 qfr[KS], dofr[KS];
-#pragma unroll
-  for (int s = 0; s < KS; ++s) {
-    qfr[s] = *reinterpret_cast<const uintx4*>(qp + 16 * s + 8 * g);
-    dofr[s] = *reinterpret_cast<const uintx4*>(gp + 16 * s + 8 * g);
-  }
   // a query without any unmasked key has lse = -inf: every P of its row must come out as 0
-  const float lse_q = prm.lse[(int64_t)bh * prm.N + qrow];
   float lse2 = EW && lse_q == -INFINITY ? INFINITY : lse_q * kLog2e;
   // delta = rowsum(O * dO) (fa2_bwd.py:17): the lane holds one half of its query's row of dO, its neighbour 32
   // lanes on the other half.  Also kept for the dK/dV kernel, which needs it by key tile.
   float dlt;
   {
-    const unsigned short* op = (const unsigned short*)prm.o + b * prm.os[0] + h * prm.os[1] + qrow * prm.os[2];
     float acc = 0.f;
 #pragma unroll
-    for (int s = 0; s < KS; ++s) acc = dot8<BF16>(*reinterpret_cast<const uintx4*>(op + 16 * s + 8 * g), dofr[s], acc);
+    for (int s = 0; s < KS; ++s) acc = dot8<BF16>(ofr[s], dofr[s], acc);
     dlt = acc + __shfl_xor(acc, 32);
     if (chunk == 0 && g == 0) prm.delta[(int64_t)bh * prm.N + qrow] = dlt;
   }
@@ -321,15 +325,12 @@ __global__ __launch_bounds__(128, D == 256 ? 1 : 2) void dq_kernel(const BwdPara
                          dqacc[db][4 * i4 + 2], dqacc[db][4 * i4 + 3]);
     return;
   }
-  const int64_t hoff = b * prm.dqs[0] + h * prm.dqs[1];
-  void* base = prm.out_f32 ? (void*)((float*)prm.dq + hoff) : (void*)((unsigned short*)prm.dq + hoff);
-#pragma unroll
-  for (int db = 0; db < DB; ++db)
-#pragma unroll
-    for (int i4 = 0; i4 < 4; ++i4)
-      store_out4<BF16>(base, qrow * prm.dqs[2] + 32 * db + 8 * i4 + 4 * g, prm.out_f32, dqacc[db][4 * i4] * prm.sm_scale,
-                       dqacc[db][4 * i4 + 1] * prm.sm_scale, dqacc[db][4 * i4 + 2] * prm.sm_scale,
-                       dqacc[db][4 * i4 + 3] * prm.sm_scale);
+  // dQ rows leave through this wavefront's stage of the (now idle) tile buffers
+  static_assert(rows_out_bytes(D, true) <= C::STAGE_BYTES, "a stage holds a wavefront's 32 result rows");
+  __syncthreads();           // the other wavefront has left its last step
+  const float sc = prm.sm_scale;
+  rows_out<BF16, D>(lds + wv * C::STAGE_BYTES, prm.dq, b * prm.dqs[0] + h * prm.dqs[1] + ((int64_t)m * 64 + 32 * wv) * prm.dqs[2],
+                    prm.dqs[2], prm.out_f32, lane, [&](int db, int i) { return dqacc[db][i] * sc; });
 }
 
 // ---------------------------------------------------------------------------------------
@@ -694,6 +695,17 @@ __global__ __launch_bounds__(256, 2) void dkdv4_kernel(const BwdParams prm) {
   const int mh = (prm.Bm > 1 ? b : 0) * prm.Hm + (prm.Hm > 1 ? h : 0);
   const cint_ptr_t cp = (cint_ptr_t)(uintptr_t)(prm.col_ptr + (int64_t)mh * nb);
   const cint_ptr_t rows = (cint_ptr_t)(uintptr_t)prm.row_idx;
+  // The K and V rows this wavefront owns for the whole walk depend on the block index only: asked for first, they
+  // travel while the list is looked up and the first tiles are requested.
+  const int64_t krow = (int64_t)n * 64 + 32 * kh + ln;
+  const unsigned short* kp = (const unsigned short*)prm.k + b * prm.ks[0] + h * prm.ks[1] + krow * prm.ks[2];
+  const unsigned short* vp = (const unsigned short*)prm.v + b * prm.vs[0] + h * prm.vs[1] + krow * prm.vs[2];
+  uintx4 kfr[KS], vfr[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    kfr[s] = *reinterpret_cast<const uintx4*>(kp + 16 * s + 8 * g);
+    vfr[s] = *reinterpret_cast<const uintx4*>(vp + 16 * s + 8 * g);
+  }
   int u0, u1;
   {
     const int t0 = cp[n], len = cp[n + 1] - t0;                // this workgroup's share of the column's list
@@ -728,15 +740,6 @@ __global__ __launch_bounds__(256, 2) void dkdv4_kernel(const BwdParams prm) {
   };
   if (u0 < u1) { ask_stats(u0); issue(u0, 0); }
 
-  const int64_t krow = (int64_t)n * 64 + 32 * kh + ln;
-  const unsigned short* kp = (const unsigned short*)prm.k + b * prm.ks[0] + h * prm.ks[1] + krow * prm.ks[2];
-  const unsigned short* vp = (const unsigned short*)prm.v + b * prm.vs[0] + h * prm.vs[1] + krow * prm.vs[2];
-  uintx4 kfr[KS], vfr[KS];
-#pragma unroll
-  for (int s = 0; s < KS; ++s) {
-    kfr[s] = *reinterpret_cast<const uintx4*>(kp + 16 * s + 8 * g);
-    vfr[s] = *reinterpret_cast<const uintx4*>(vp + 16 * s + 8 * g);
-  }
 #pragma unroll
   for (int s = 0; s < KS; ++s) { settle(kfr[s]); settle(vfr[s]); }   // K and V are there: no waits for them in the loop
   const float qk_scale = prm.qk_scale;
@@ -862,19 +865,17 @@ __global__ __launch_bounds__(256, 2) void dkdv4_kernel(const BwdParams prm) {
       }
     return;
   }
-  const int64_t koffh = b * prm.dks[0] + h * prm.dks[1], voffh = b * prm.dvs[0] + h * prm.dvs[1];
-  void* kbase = prm.out_f32 ? (void*)((float*)prm.dk + koffh) : (void*)((unsigned short*)prm.dk + koffh);
-  void* vbase = prm.out_f32 ? (void*)((float*)prm.dv + voffh) : (void*)((unsigned short*)prm.dv + voffh);
-#pragma unroll
-  for (int db = 0; db < DBW; ++db)
-#pragma unroll
-    for (int i4 = 0; i4 < 4; ++i4) {
-      const int col = 32 * (DBW * dh + db) + 8 * i4 + 4 * g;
-      store_out4<BF16>(kbase, krow * prm.dks[2] + col, prm.out_f32, dkacc[db][4 * i4] * prm.sm_scale, dkacc[db][4 * i4 + 1] * prm.sm_scale,
-                       dkacc[db][4 * i4 + 2] * prm.sm_scale, dkacc[db][4 * i4 + 3] * prm.sm_scale);
-      store_out4<BF16>(vbase, krow * prm.dvs[2] + col, prm.out_f32, dvacc[db][4 * i4], dvacc[db][4 * i4 + 1], dvacc[db][4 * i4 + 2],
-                       dvacc[db][4 * i4 + 3]);
-    }
+  // the wavefront's 32 x 64 blocks of dK and dV leave through a stretch of the (now idle) tile stages and exchange area
+  constexpr int OUT_BYTES = rows_out_bytes(32 * DBW, true);
+  static_assert(4 * 2 * OUT_BYTES <= DKDV4_LDS_BYTES, "room for dK and dV of four wavefronts");
+  __syncthreads();           // everybody has left the last step
+  unsigned char* mine = lds + wv * 2 * OUT_BYTES;
+  const int64_t r0 = (int64_t)n * 64 + 32 * kh;
+  const float sc = prm.sm_scale;
+  rows_out<BF16, 32 * DBW>(mine, prm.dk, b * prm.dks[0] + h * prm.dks[1] + r0 * prm.dks[2] + 32 * DBW * dh, prm.dks[2],
+                           prm.out_f32, lane, [&](int db, int i) { return dkacc[db][i] * sc; });
+  rows_out<BF16, 32 * DBW>(mine + OUT_BYTES, prm.dv, b * prm.dvs[0] + h * prm.dvs[1] + r0 * prm.dvs[2] + 32 * DBW * dh, prm.dvs[2],
+                           prm.out_f32, lane, [&](int db, int i) { return dvacc[db][i]; });
 }
 
 // ---------------------------------------------------------------------------------------

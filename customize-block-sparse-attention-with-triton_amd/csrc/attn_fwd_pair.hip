@@ -57,6 +57,15 @@ __global__ __launch_bounds__(128, D == 128 ? 2 : 1) void fwd_pair_kernel(const F
   const int b = bh / prm.H, h = bh % prm.H;
   const int mh = (prm.Bm > 1 ? b : 0) * prm.Hm + (prm.Hm > 1 ? h : 0);
   const cint_ptr_t rp = (cint_ptr_t)(uintptr_t)(prm.row_ptr + (int64_t)mh * nb);
+  // Q of this lane's query (second operand of S^T = K Q^T) depends on the block index only: asked for first, it
+  // travels while the list is looked up and the first tiles are requested.
+  const int64_t qrow = (int64_t)m * 64 + 32 * w + ln;          // this lane's query
+  uintx4 qf[1][KS];
+  {
+    const unsigned short* qp = (const unsigned short*)prm.q + b * prm.qs[0] + h * prm.qs[1] + qrow * prm.qs[2];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) qf[0][s] = *reinterpret_cast<const uintx4*>(qp + 16 * s + 8 * g);
+  }
   int t0 = rp[m], t1 = rp[m + 1];
   if (prm.split > 1) {                           // this workgroup's share of the row block's list
     const int len = t1 - t0;
@@ -65,7 +74,6 @@ __global__ __launch_bounds__(128, D == 128 ? 2 : 1) void fwd_pair_kernel(const F
     if (t0 == t1) return;                        // (pair_sum_parts_kernel knows which shares are empty)
   }
   void* obase = out_base(prm, b, h);
-  const int64_t qrow = (int64_t)m * 64 + 32 * w + ln;          // this lane's query
   if (t0 == t1) {                                // no kept tile: O = 0, lse = -inf
 #pragma unroll
     for (int db = 0; db < DB; ++db)
@@ -84,7 +92,6 @@ __global__ __launch_bounds__(128, D == 128 ? 2 : 1) void fwd_pair_kernel(const F
   const unsigned lds_v_addr = lds_k_addr + TILE_BYTES;
   const unsigned lds_bits_addr = lds_k_addr + 2 * TILE_BYTES;
 
-  const unsigned short* qg = (const unsigned short*)prm.q + b * prm.qs[0] + h * prm.qs[1];
   const unsigned short* kg = (const unsigned short*)prm.k + b * prm.ks[0] + h * prm.ks[1];
   const unsigned short* vg = (const unsigned short*)prm.v + b * prm.vs[0] + h * prm.vs[1];
   const float qk_scale = prm.qk_scale;
@@ -97,11 +104,6 @@ __global__ __launch_bounds__(128, D == 128 ? 2 : 1) void fwd_pair_kernel(const F
     if constexpr (EW) c |= (int)((cbyte_ptr_t)(uintptr_t)prm.tile_partial)[t] << 30;
     return c;
   };
-  for (int i = threadIdx.x; i < t1 - t0 && i < PAIR_COLS_CAP; i += 128) {
-    int c = prm.col_idx[t0 + i];
-    if constexpr (EW) c |= (int)prm.tile_partial[t0 + i] << 30;
-    lcols[i] = c;
-  }
   constexpr int COL_MASK = 0x3fffffff;
   auto col_of = [&](int t) { return t - t0 < PAIR_COLS_CAP ? lcols[t - t0] : flagged_col(t); };
 
@@ -170,16 +172,14 @@ __global__ __launch_bounds__(128, D == 128 ? 2 : 1) void fwd_pair_kernel(const F
   const int vkey0 = 4 * (vblk >> 1) + (vs_ >> 2), vcol0 = 16 * (vblk & 1) + 4 * (vs_ & 3);
   const uintx4 ones_frag = {g == 0 ? 0x3c003c00u : 0u, 0u, 0u, 0u};
 
-  // first tile's copies, then Q (this lane's query: second operand of S^T = K Q^T)
-  __syncthreads();                                  // lcols
-  int cx = __builtin_amdgcn_readfirstlane(col_of(t0));
+  // first tile's copies (its column from one scalar load), then the column list into LDS
+  int cx = flagged_col(t0);
   k_copy(cx & COL_MASK, t0);
   v_copy(cx & COL_MASK);
-  uintx4 qf[1][KS];
-  {
-    const unsigned short* qp = qg + qrow * prm.qs[2];
-#pragma unroll
-    for (int s = 0; s < KS; ++s) qf[0][s] = *reinterpret_cast<const uintx4*>(qp + 16 * s + 8 * g);
+  for (int i = threadIdx.x; i < t1 - t0 && i < PAIR_COLS_CAP; i += 128) {
+    int c = prm.col_idx[t0 + i];
+    if constexpr (EW) c |= (int)prm.tile_partial[t0 + i] << 30;
+    lcols[i] = c;
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0), visible to the compiler: Q and the first tiles
   if constexpr (FOLD) {
@@ -200,7 +200,7 @@ __global__ __launch_bounds__(128, D == 128 ? 2 : 1) void fwd_pair_kernel(const F
   uintx4 mfrag = {0u, 0u, 0u, 0u};
   bool fresh = true;
   int any_m = 0;     // (wave-uniform) some lane's reference exponent is not zero: the extra contraction slice is needed
-  __syncthreads();                                  // both halves of K(t0) and V(t0) are in LDS
+  __syncthreads();                                  // both halves of K(t0) and V(t0) and the column list are in LDS
 
   for (int t = t0; t < t1; ++t) {
     const bool has1 = t + 1 < t1;
@@ -343,12 +343,11 @@ __global__ __launch_bounds__(128, D == 128 ? 2 : 1) void fwd_pair_kernel(const F
     return;
   }
   const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
-#pragma unroll
-  for (int db = 0; db < DB; ++db)
-#pragma unroll
-    for (int i4 = 0; i4 < 4; ++i4)
-      store_out4<BF16>(obase, qrow * prm.os[2] + 32 * db + 8 * i4 + 4 * g, prm.out_f32, oacc[db][0][4 * i4] * inv,
-                       oacc[db][0][4 * i4 + 1] * inv, oacc[db][0][4 * i4 + 2] * inv, oacc[db][0][4 * i4 + 3] * inv);
+  // the wavefront's 32 rows of O leave through its half of the (now idle) LDS
+  static_assert(2 * rows_out_bytes(D, true) <= pair_lds_bytes<D>(), "room for the result rows of both wavefronts");
+  __syncthreads();           // the other wavefront has left its last tile
+  rows_out<BF16, D>(lds + w * rows_out_bytes(D, true), obase, ((int64_t)m * 64 + 32 * w) * prm.os[2], prm.os[2], prm.out_f32,
+                    lane, [&](int db, int i) { return oacc[db][0][i] * inv; });
   if (prm.lse != nullptr && g == 0)
     prm.lse[(int64_t)bh * prm.N + qrow] =
         lsum > 0.f ? (m_i + __builtin_amdgcn_logf(lsum)) * 0.6931471805599453f : -INFINITY;

@@ -156,6 +156,55 @@ __device__ __forceinline__ void store_out4(void* obase, int64_t elem_off, bool o
 }
 
 
+// The 32 result rows of a wavefront leave through LDS, so that a store instruction writes 16 bytes per lane with
+// consecutive lanes along a row (whole rows, or 128-byte stretches of them) instead of 8 or 16 bytes in each of
+// 32 rows.  The lane holds, of row `ln` of the 32, value(db, i) for column 32 db + 8 (i / 4) + 4 g + i % 4 (the
+// layout in which a 32x32 MFMA result holds its rows), db < NCOL / 32.
+// stage: ROWS_OUT_BYTES(NCOL, out_f32) bytes of LDS that only this wavefront touches (its LDS accesses are executed
+// in order, so the reads below see the writes above them without a barrier).
+// out + elem_off: row 0, first of the NCOL columns; row_stride in elements; rows 16-byte aligned.
+__host__ __device__ constexpr int rows_out_bytes(int ncol, bool out_f32) { return 32 * (ncol * (out_f32 ? 4 : 2) + 16); }
+template <bool BF16, int NCOL, typename F>
+__device__ __forceinline__ void rows_out(unsigned char* stage, void* out, int64_t elem_off, int64_t row_stride,
+                                         bool out_f32, int lane, F&& value) {
+  const int ln = lane & 31, g = lane >> 5;
+  if (out_f32) {
+    constexpr int PITCH = NCOL * 4 + 16, LPR = NCOL / 4, RPI = 64 / LPR;   // lanes per row, rows per instruction
+#pragma unroll
+    for (int db = 0; db < NCOL / 32; ++db)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const floatx4 w = {value(db, 4 * i4), value(db, 4 * i4 + 1), value(db, 4 * i4 + 2), value(db, 4 * i4 + 3)};
+        *reinterpret_cast<floatx4*>(stage + ln * PITCH + (32 * db + 8 * i4 + 4 * g) * 4) = w;
+      }
+    __builtin_amdgcn_wave_barrier();
+    float* o = (float*)out + elem_off;
+#pragma unroll
+    for (int it = 0; it < 32 / RPI; ++it) {
+      const int r = it * RPI + lane / LPR, c = lane % LPR;
+      const floatx4 w = *reinterpret_cast<const floatx4*>(stage + r * PITCH + 16 * c);
+      *reinterpret_cast<floatx4*>(o + r * row_stride + 4 * c) = w;
+    }
+  } else {
+    constexpr int PITCH = NCOL * 2 + 16, LPR = NCOL / 8, RPI = 64 / LPR;
+#pragma unroll
+    for (int db = 0; db < NCOL / 32; ++db)
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const uintx2 w = {pack2<BF16>(value(db, 4 * i4), value(db, 4 * i4 + 1)), pack2<BF16>(value(db, 4 * i4 + 2), value(db, 4 * i4 + 3))};
+        *reinterpret_cast<uintx2*>(stage + ln * PITCH + (32 * db + 8 * i4 + 4 * g) * 2) = w;
+      }
+    __builtin_amdgcn_wave_barrier();
+    unsigned short* o = (unsigned short*)out + elem_off;
+#pragma unroll
+    for (int it = 0; it < 32 / RPI; ++it) {
+      const int r = it * RPI + lane / LPR, c = lane % LPR;
+      const uintx4 w = *reinterpret_cast<const uintx4*>(stage + r * PITCH + 16 * c);
+      *reinterpret_cast<uintx4*>(o + r * row_stride + 8 * c) = w;
+    }
+  }
+}
+
 // Partial results cross workgroups (and the L2 slices of different XCDs) inside one launch:
 // they are written and read with device-scope accesses, which go to the point of coherence.
 __device__ __forceinline__ void coherent_store(float* p, float v) {
