@@ -96,7 +96,7 @@ void fwd_kernel(const FwdParams prm) {
   // block's end only from very close; short ranges are cut on the plain tile axis and their boundaries move to
   // the nearer end of a row block from up to SNAP tiles away (row blocks of up to 2 SNAP tiles are never shared).
 #ifndef LONG_GAP
-#define LONG_GAP 8
+#define LONG_GAP 12
 #define LONG_SNAP 2
 #endif
   const bool long_ranges = !ROWS && ((int64_t)hs.T >= (int64_t)EQUAL_SPLIT_BELOW * hs.Peff || hs.Peff >= 3 * nb);   // (or row blocks much longer than the ranges)
