@@ -869,13 +869,17 @@ __global__ __launch_bounds__(256, 2) void dkdv4_kernel(const BwdParams prm) {
   constexpr int OUT_BYTES = rows_out_bytes(32 * DBW, true);
   static_assert(4 * 2 * OUT_BYTES <= DKDV4_LDS_BYTES, "room for dK and dV of four wavefronts");
   __syncthreads();           // everybody has left the last step
+  // (the lane index as a value the compiler cannot trace back: the per-lane addresses of the stores below would
+  // otherwise be computed before the walk and held, or spilled, through it)
+  int lane_out = lane;
+  asm volatile("" : "+v"(lane_out));
   unsigned char* mine = lds + wv * 2 * OUT_BYTES;
   const int64_t r0 = (int64_t)n * 64 + 32 * kh;
   const float sc = prm.sm_scale;
   rows_out<BF16, 32 * DBW>(mine, prm.dk, b * prm.dks[0] + h * prm.dks[1] + r0 * prm.dks[2] + 32 * DBW * dh, prm.dks[2],
-                           prm.out_f32, lane, [&](int db, int i) { return dkacc[db][i] * sc; });
+                           prm.out_f32, lane_out, [&](int db, int i) { return dkacc[db][i] * sc; });
   rows_out<BF16, 32 * DBW>(mine + OUT_BYTES, prm.dv, b * prm.dvs[0] + h * prm.dvs[1] + r0 * prm.dvs[2] + 32 * DBW * dh, prm.dvs[2],
-                           prm.out_f32, lane, [&](int db, int i) { return dvacc[db][i]; });
+                           prm.out_f32, lane_out, [&](int db, int i) { return dvacc[db][i]; });
 }
 
 // ---------------------------------------------------------------------------------------
