@@ -164,6 +164,38 @@ def test_packed_qkv_layout_is_kept(dev, out_fp32):
         assert ma <= 2e-2 and rl <= 1e-3
 
 
+@pytest.mark.parametrize("out_fp32", [False, True])
+def test_packed_qkv_layout_d128_whole_lists(dev, out_fp32):
+    """Packed [B, N, 3, H, D] inputs at D = 128 with enough row blocks that every list belongs to one workgroup: the
+    pair forward kernel, dq_kernel and dkdv4_kernel then write their result rows themselves, through LDS and through
+    the strides of the results.  Two heads against the oracle, all heads against the same call on contiguous copies."""
+    import fa2_custom_mask as fm
+    B, H, N, D, nb = 2, 8, 4096, 128, 64
+    g = torch.Generator().manual_seed(43)
+    qkv = torch.randn(B, N, 3, H, D, generator=g).to(torch.bfloat16)
+    do = torch.randn(B, N, H, D, generator=g).to(torch.bfloat16)
+    mask = uniform_block_mask(1, 1, nb, 0.3, 11)
+    sc = 1.0 / np.sqrt(D)
+    qkv_d, do_d = qkv.to(dev), do.to(dev)
+    q, k, v = [qkv_d[:, :, i].transpose(1, 2) for i in range(3)]
+    res = fm.attention_forward_backward(q, k, v, mask.to(dev), sc, do_d.transpose(1, 2), out_fp32=out_fp32)
+    want = torch.empty_like(q, dtype=torch.float32 if out_fp32 else torch.bfloat16).stride()
+    for t in (res[0], res[2], res[3], res[4]):
+        assert t.stride() == want == (N * H * D, D, H * D, 1)
+    ref = fm.attention_forward_backward(q.contiguous(), k.contiguous(), v.contiguous(), mask.to(dev), sc,
+                                        do_d.transpose(1, 2).contiguous(), out_fp32=out_fp32)
+    for a_, b_ in zip(res, ref):
+        assert torch.equal(a_, b_)                        # the layout of the results changes no value
+    for (b, h) in ((0, 1), (1, 6)):
+        qh, kh, vh = [f32(qkv[b:b + 1, :, i, h:h + 1].transpose(1, 2).contiguous()) for i in range(3)]
+        doh = f32(do[b:b + 1, :, h:h + 1].transpose(1, 2).contiguous())
+        o_r = orc.naive_attention(qh, kh, vh, mask.numpy(), sc)
+        dq_r, dk_r, dv_r, _ = orc.attention_backward(qh, kh, vh, mask.numpy(), sc, doh)
+        for got, r in ((res[0], o_r), (res[2], dq_r), (res[3], dk_r), (res[4], dv_r)):
+            ma, rl = errors(got[b:b + 1, h:h + 1], r)
+            assert ma <= 3e-2 and rl <= (1e-3 if out_fp32 else 3e-3)
+
+
 def test_packed_qkv_split_lists(dev):
     """The same for a single long head, whose row and column lists are walked by several workgroups (the
     gradients are then summed from fp32 parts by a kernel of its own, which writes through the strides)."""
