@@ -53,10 +53,7 @@ template <int D> struct FwdCfg {
   static constexpr int ROUNDS = D / R;
   static constexpr int QPW = (R / 4) / NW;                  // output quads per wavefront and round
   static constexpr int SHORT_ROW = 6 * NW;                  // row blocks up to this many tiles may go to one wavefront
-#ifndef SNAP_TILES
-#define SNAP_TILES 8
-#endif
-  static constexpr int SNAP = SNAP_TILES;                   // a range boundary this close to an end of its row block moves there
+  static constexpr int SNAP = 16;                           // short ranges: a boundary at least this close to an end of its row block moves there
 };
 
 // DT: 0 fp16; 1 bf16 with P rounded to fp16 (V fragments converted); 2 bf16 with P rounded to bf16.
@@ -94,13 +91,17 @@ void fwd_kernel(const FwdParams prm) {
   HeadSplit hs = head_split(rp, nb, prm.W, MIN_TILES, prm.first_ids > bh ? (prm.first_ids - bh + BH - 1) / BH : 0, 0);
   // Long ranges (the regime of the weighted shares) are cut on the axis with gaps and boundaries move to a row
   // block's end only from very close; short ranges are cut on the plain tile axis and their boundaries move to
-  // the nearer end of a row block from up to SNAP tiles away (row blocks of up to 2 SNAP tiles are never shared).
+  // the nearer end of a row block from up to half a range (and at least SNAP tiles) away: a row block is shared
+  // only where a boundary falls into its middle, row blocks of up to a range's length or 2 SNAP tiles never (N = 17536,
+  // one head, against 8 tiles for every head: keep 0.15 36.0 -> 31.4 us, keep 0.2 40.0 -> 34.6, keep 0.25 43.2 -> 39.8,
+  // keep 0.05 21.8 -> 20.2, keep 0.1 25.8 -> 25.1; keep 0.35 and above, other sizes: +-1 %).
 #ifndef LONG_GAP
 #define LONG_GAP 12
 #define LONG_SNAP 2
 #endif
   const bool long_ranges = !ROWS && ((int64_t)hs.T >= (int64_t)EQUAL_SPLIT_BELOW * hs.Peff || hs.Peff >= 3 * nb);   // (or row blocks much longer than the ranges)
-  const int snap = long_ranges ? LONG_SNAP : C::SNAP;
+  const int half_range = hs.T / (2 * (hs.Peff > 0 ? hs.Peff : 1)) + 1;
+  const int snap = long_ranges ? LONG_SNAP : (half_range > C::SNAP ? half_range : C::SNAP);
   if (long_ranges) { hs.gap = LONG_GAP; hs.X = (int64_t)hs.T + (int64_t)LONG_GAP * nb; }
   // Which range this workgroup takes (launches with few heads and long ranges): the ranges of a head start at
   // all phases of a row, and workgroups that share an XCD, hence an L2, get ranges of like phase, so that they
@@ -588,10 +589,10 @@ void fwd_kernel(const FwdParams prm) {
     // K / V buffer has been issued; no copy is issued across the merge of a row block, which
     // borrows both buffers of every wavefront (one exchange round for the whole accumulator).
     // first row block of the range: largest r with rp[r] <= g0 < rp[r+1]
-    // A range boundary within SNAP tiles of an end of the row block it falls in moves to that end
+    // A range boundary within `snap` tiles of an end of the row block it falls in moves to that end
     // (the nearer one): sharing a row block costs a merge, a published part and a pull, several
-    // tiles' worth each, and row blocks of up to 2 SNAP tiles are never shared.  Every workgroup
-    // applies the same rule to both of its boundaries, so the ranges still tile the list.
+    // tiles' worth each, and row blocks of up to 2 `snap` tiles are never shared.  Every workgroup
+    // applies the same rule with the same distance to both of its boundaries, so the ranges still tile the list.
     int r;
     {
       // the row blocks in which the two ends of the range lie (positions behind a row block's tiles count as
