@@ -53,7 +53,7 @@ template <int D> struct FwdCfg {
   static constexpr int ROUNDS = D / R;
   static constexpr int QPW = (R / 4) / NW;                  // output quads per wavefront and round
   static constexpr int SHORT_ROW = 6 * NW;                  // row blocks up to this many tiles may go to one wavefront
-  static constexpr int SNAP = 16;                           // short ranges: a boundary at least this close to an end of its row block moves there
+  static constexpr int SNAP = WG_PER_CU > 1 ? 16 : 8;       // short ranges: a boundary at least this close to an end of its row block moves there
 };
 
 // DT: 0 fp16; 1 bf16 with P rounded to fp16 (V fragments converted); 2 bf16 with P rounded to bf16.
@@ -100,8 +100,10 @@ void fwd_kernel(const FwdParams prm) {
 #define LONG_SNAP 2
 #endif
   const bool long_ranges = !ROWS && ((int64_t)hs.T >= (int64_t)EQUAL_SPLIT_BELOW * hs.Peff || hs.Peff >= 3 * nb);   // (or row blocks much longer than the ranges)
+  // (D = 128, one workgroup per compute unit and tiles twice as long: sharing a row block is cheaper against the
+  // imbalance it avoids; 8 tiles for every head.  Half a range there: keep 0.1 87 -> 98 us, keep 0.15 107 -> 129 us.)
   const int half_range = hs.T / (2 * (hs.Peff > 0 ? hs.Peff : 1)) + 1;
-  const int snap = long_ranges ? LONG_SNAP : (half_range > C::SNAP ? half_range : C::SNAP);
+  const int snap = long_ranges ? LONG_SNAP : (C::WG_PER_CU > 1 && half_range > C::SNAP ? half_range : C::SNAP);
   if (long_ranges) { hs.gap = LONG_GAP; hs.X = (int64_t)hs.T + (int64_t)LONG_GAP * nb; }
   // Which range this workgroup takes (launches with few heads and long ranges): the ranges of a head start at
   // all phases of a row, and workgroups that share an XCD, hence an L2, get ranges of like phase, so that they
