@@ -132,8 +132,9 @@ __global__ __launch_bounds__(256) void fill_rows_kernel(const uint8_t* __restric
 // LDS with one bit per byte: thread r then finds the start of row r as the count in front of the segment that
 // holds byte r * nb plus the set bits of that segment below it.  Lengths and the rows' positions in `groups`
 // follow from the starts after a second scan over the non-empty flags.
-// fill_rows_kernel then writes col_idx and groups with the whole GPU (one workgroup writing 75 000 scattered
-// entries takes 50 us).
+// The same launch writes col_idx and groups: one workgroup writing 75 000 scattered entries would take 36-50 us, so
+// for masks of more than LISTS_FILL_MAX tiles the launch has 64 workgroups, each of which counts and scans the
+// whole mask for itself (75 KB from the L2) and fills a 64th of the entries.
 // ---------------------------------------------------------------------------------------
 constexpr int LISTS_ONE_MAX_ROWS = 1023, LISTS_ONE_MAX_SEG = 256;
 
@@ -159,10 +160,9 @@ __device__ __forceinline__ int block_inclusive_sum(int v, int* s_w, int* total) 
   return v + before;
 }
 
-// FILL: the same workgroup also writes col_idx and groups, every thread the entries of its own segment (masks
-// of up to LISTS_FILL_MAX tiles, where one workgroup's scattered stores cost less than a second launch).
+// The kernel also writes col_idx and groups, every thread the entries of its own segment: with one workgroup for
+// masks of up to LISTS_FILL_MAX tiles, with several for larger ones (see below).
 constexpr int LISTS_FILL_MAX = 16384;
-template <bool FILL>
 __global__ __launch_bounds__(1024) void count_scan_kernel(const uint8_t* __restrict__ block, int rows, int nb,
                                                           int seg, int32_t* __restrict__ row_ptr,
                                                           int32_t* __restrict__ gidx, int32_t* __restrict__ counts,
@@ -217,8 +217,8 @@ __global__ __launch_bounds__(1024) void count_scan_kernel(const uint8_t* __restr
         const unsigned m = below <= 0 ? 0u : below >= 32 ? ~0u : (1u << below) - 1u;
         start += __popc(s_bits[t][w] & m);
       }
-      row_ptr[tid] = start;
-    } else {
+      if (blockIdx.x == 0) row_ptr[tid] = start;
+    } else if (blockIdx.x == 0) {
       row_ptr[rows] = kept; counts[1] = kept;
     }
     s_start[tid] = start;
@@ -227,24 +227,56 @@ __global__ __launch_bounds__(1024) void count_scan_kernel(const uint8_t* __restr
   const int len = tid < rows ? s_start[tid + 1] - s_start[tid] : 0;
   int ngroups;
   const int gi = block_inclusive_sum(len > 0 ? 1 : 0, s_w, &ngroups) - (len > 0 ? 1 : 0);
-  if (tid < rows) gidx[tid] = gi;
-  if (tid == 0) counts[0] = ngroups;
-  if constexpr (FILL) {
+  if (blockIdx.x == 0) {
+    if (tid < rows) gidx[tid] = gi;
+    if (tid == 0) counts[0] = ngroups;
+  }
+  if (gridDim.x == 1) {
     // entry number s_off[tid] + k of the list is the k-th set byte of this thread's segment: its column block
     int pos = s_off[tid];
+    int col = base % nb;                          // column block of the segment's first byte
 #pragma unroll
     for (int w = 0; w < WORDS; ++w) {
       unsigned b = bits[w];
+      int at = 0;                                 // bit position that `col` belongs to
       while (b != 0u) {
         const int bit = __ffs(b) - 1;
         b &= b - 1u;
-        col_idx[pos++] = (base + 32 * w + bit) % nb;
+        col += bit - at; at = bit;
+        while (col >= nb) col -= nb;
+        col_idx[pos++] = col;
       }
+      col += 32 - at;
+      while (col >= nb) col -= nb;
     }
     if (groups != nullptr && len > 0) {
       const int bh = tid / nb;
       int32_t* g = groups + (int64_t)gi * 5;
       g[0] = bh / H; g[1] = bh % H; g[2] = tid % nb; g[3] = s_start[tid]; g[4] = len;
+    }
+  } else {
+    // Larger masks: several workgroups, each of which has counted and scanned the whole mask for itself (it sits in
+    // the L2) and now fills its share of the rows, one wavefront per row (ballot and rank, as fill_rows_kernel):
+    // one workgroup alone would spend 36 us on the scattered stores of 75 000 entries.
+    if (tid < rows) s_off[tid] = gi;              // (the segments' offsets are no longer needed)
+    __syncthreads();
+    const int lane = tid & 63, nw = (int)gridDim.x * 16;
+    for (int row = (int)blockIdx.x * 16 + (tid >> 6); row < rows; row += nw) {
+      const uint8_t* p = block + (int64_t)row * nb;
+      const int start = s_start[row];
+      int pos = start;
+      for (int n0 = 0; n0 < nb; n0 += 64) {
+        const int n = n0 + lane;
+        const bool keep = n < nb && p[n] != 0;
+        const unsigned long long bal = __ballot(keep);
+        if (keep) col_idx[pos + __popcll(bal & ((1ull << lane) - 1ull))] = n;
+        pos += __popcll(bal);
+      }
+      if (groups != nullptr && lane == 0 && pos > start) {
+        const int bh = row / nb;
+        int32_t* g = groups + (int64_t)s_off[row] * 5;
+        g[0] = bh / H; g[1] = bh % H; g[2] = row % nb; g[3] = start; g[4] = pos - start;
+      }
     }
   }
 }
@@ -506,13 +538,14 @@ int launch_block_mask_to_lists(const uint8_t* block, int Bm, int Hm, int nb, int
   const dim3 grid((rows + 3) / 4);
   if (contiguous && rows <= LISTS_ONE_MAX_ROWS && total <= 1024 * LISTS_ONE_MAX_SEG) {
     const int seg = (((int)total + 1023) / 1024 + 15) / 16 * 16;
-    if (total <= LISTS_FILL_MAX) {      // (the whole call in one launch)
-      hipLaunchKernelGGL((count_scan_kernel<true>), dim3(1), dim3(1024), 0, st, block, rows, nb, seg, row_ptr, gidx, counts,
-                         Hm, col_idx, groups);
-      return launch_status();
-    }
-    hipLaunchKernelGGL((count_scan_kernel<false>), dim3(1), dim3(1024), 0, st, block, rows, nb, seg, row_ptr, gidx, counts,
-                       Hm, col_idx, groups);
+#ifndef LISTS_FILL_WGS
+#define LISTS_FILL_WGS 32
+#endif
+    // the whole call in one launch: one workgroup for small masks, LISTS_FILL_WGS for larger ones (each counts and
+    // scans for itself and fills its share)
+    hipLaunchKernelGGL(count_scan_kernel, dim3(total <= LISTS_FILL_MAX ? 1 : LISTS_FILL_WGS), dim3(1024), 0, st, block,
+                       rows, nb, seg, row_ptr, gidx, counts, Hm, col_idx, groups);
+    return launch_status();
   } else {
     hipLaunchKernelGGL(count_rows_kernel, grid, dim3(256), 0, st, block, rows, nb, Hm, sb, sh, sm, sn, cnt);
     hipLaunchKernelGGL(scan_rows_kernel, dim3(1), dim3(1024), 0, st, cnt, rows, row_ptr, gidx, counts);
