@@ -104,7 +104,10 @@ void fwd_kernel(const FwdParams prm) {
   // imbalance it avoids; 8 tiles for every head.  Half a range there: keep 0.1 87 -> 98 us, keep 0.15 107 -> 129 us.)
   const int half_range = hs.T / (2 * (hs.Peff > 0 ? hs.Peff : 1)) + 1;
   const int snap = long_ranges ? LONG_SNAP : (C::WG_PER_CU > 1 && half_range > C::SNAP ? half_range : C::SNAP);
-  if (long_ranges) { hs.gap = LONG_GAP; hs.X = (int64_t)hs.T + (int64_t)LONG_GAP * nb; }
+  // (ranges that are long only against the row blocks they lie in, several to a row block: 24 positions; N = 6400
+  // dense 31.2 -> 29.0 us, where 12 are best for N = 17536 dense, 102.1 against 104.0 us)
+  const int long_gap = (int64_t)hs.T >= (int64_t)EQUAL_SPLIT_BELOW * hs.Peff ? LONG_GAP : 2 * LONG_GAP;
+  if (long_ranges) { hs.gap = long_gap; hs.X = (int64_t)hs.T + (int64_t)long_gap * nb; }
   // Which range this workgroup takes (launches with few heads and long ranges): the ranges of a head start at
   // all phases of a row, and workgroups that share an XCD, hence an L2, get ranges of like phase, so that they
   // walk the same column blocks at the same time (dense N = 17536, one head: 42 instead of 196 MB fetched from
