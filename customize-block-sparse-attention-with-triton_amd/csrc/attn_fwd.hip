@@ -103,7 +103,13 @@ void fwd_kernel(const FwdParams prm) {
   // (D = 128, one workgroup per compute unit and tiles twice as long: sharing a row block is cheaper against the
   // imbalance it avoids; 8 tiles for every head.  Half a range there: keep 0.1 87 -> 98 us, keep 0.15 107 -> 129 us.)
   const int half_range = hs.T / (2 * (hs.Peff > 0 ? hs.Peff : 1)) + 1;
-  const int snap = long_ranges ? LONG_SNAP : (C::WG_PER_CU > 1 && half_range > C::SNAP ? half_range : C::SNAP);
+  // (long ranges over short row blocks, up to 32 tiles on average: a boundary moves to the nearer end of its row block
+  // from up to half such a row block away, so that next to no row block is shared; against 2 tiles: 8 heads of
+  // N = 17536 at keep 0.05 67.9 -> 62 us, 4 heads at keep 0.1 57.9 -> 54.6 us; with longer row blocks the imbalance
+  // costs more than the sharing: keep 0.35, one head, 48.0 -> 50.4 us with 12 tiles)
+  const int avg_row = hs.T / (nb > 0 ? nb : 1);
+  const int long_snap = avg_row <= 32 ? avg_row / 2 + 1 : LONG_SNAP;
+  const int snap = long_ranges ? long_snap : (C::WG_PER_CU > 1 && half_range > C::SNAP ? half_range : C::SNAP);
   // (ranges that are long only against the row blocks they lie in, several to a row block: 24 positions; N = 6400
   // dense 31.2 -> 29.0 us, where 12 are best for N = 17536 dense, 102.1 against 104.0 us)
   const int long_gap = (int64_t)hs.T >= (int64_t)EQUAL_SPLIT_BELOW * hs.Peff ? LONG_GAP : 2 * LONG_GAP;
