@@ -85,20 +85,14 @@ void fwd_kernel(const FwdParams prm) {
   // the lists are read-only for the whole launch: constant address space => scalar loads
   const cint_ptr_t rp = (cint_ptr_t)(uintptr_t)(prm.row_ptr + (int64_t)mh * nb);
   const cint_ptr_t cols = (cint_ptr_t)(uintptr_t)prm.col_idx;
-  #ifndef MIN_TILES
-#define MIN_TILES NW
-#endif
-  HeadSplit hs = head_split(rp, nb, prm.W, MIN_TILES, prm.first_ids > bh ? (prm.first_ids - bh + BH - 1) / BH : 0, 0);
+  HeadSplit hs = head_split(rp, nb, prm.W, /*min_tiles=*/NW, prm.first_ids > bh ? (prm.first_ids - bh + BH - 1) / BH : 0, 0);
   // Long ranges (the regime of the weighted shares) are cut on the axis with gaps and boundaries move to a row
   // block's end only from very close; short ranges are cut on the plain tile axis and their boundaries move to
   // the nearer end of a row block from up to half a range (and at least SNAP tiles) away: a row block is shared
   // only where a boundary falls into its middle, row blocks of up to a range's length or 2 SNAP tiles never (N = 17536,
   // one head, against 8 tiles for every head: keep 0.15 36.0 -> 31.4 us, keep 0.2 40.0 -> 34.6, keep 0.25 43.2 -> 39.8,
   // keep 0.05 21.8 -> 20.2, keep 0.1 25.8 -> 25.1; keep 0.35 and above, other sizes: +-1 %).
-#ifndef LONG_GAP
-#define LONG_GAP 12
-#define LONG_SNAP 2
-#endif
+  constexpr int LONG_GAP = 12, LONG_SNAP = 2;
   const bool long_ranges = !ROWS && ((int64_t)hs.T >= (int64_t)EQUAL_SPLIT_BELOW * hs.Peff || hs.Peff >= 3 * nb);   // (or row blocks much longer than the ranges)
   // (D = 128, one workgroup per compute unit and tiles twice as long: sharing a row block is cheaper against the
   // imbalance it avoids; 8 tiles for every head.  Half a range there: keep 0.1 87 -> 98 us, keep 0.15 107 -> 129 us.)

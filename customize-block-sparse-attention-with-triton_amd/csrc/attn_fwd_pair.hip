@@ -18,11 +18,9 @@
 #include "fwd_tile.h"
 #include "kernel_util.h"
 
-#ifndef PAIR_EARLY_V
-#define PAIR_EARLY_V 1   // largest number of fragment portions (head dimension / 128) for which V is read early
-#endif
 namespace bsattn {
 
+constexpr int PAIR_EARLY_V = 1;   // largest number of fragment portions (head dimension / 128) for which V is read early
 constexpr int PAIR_COLS_CAP = 1024;                               // column indices of the row block kept in LDS
 template <int D> constexpr int pair_lds_bytes() { return 2 * 64 * 2 * D + 512 + PAIR_COLS_CAP * 4; }   // K tile, V tile, mask words, columns
 

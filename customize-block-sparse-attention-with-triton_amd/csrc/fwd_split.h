@@ -9,6 +9,8 @@ namespace bsattn {
 // second).  The first `fast` ranges of a head therefore receive tiles in the proportion
 // WEIGHT_FAST : WEIGHT_SLOW to the others.
 constexpr int WEIGHT_FAST = 3, WEIGHT_SLOW = 2;
+// Heads with fewer tiles per range than this are cut into equal shares.
+constexpr int EQUAL_SPLIT_BELOW = 48;
 
 struct HeadSplit {
   int lo;     // first tile of the head in the global list
@@ -38,9 +40,6 @@ __device__ __forceinline__ HeadSplit head_split(Ptr rp, int nb, int P, int min_t
   const int want = (s.T + min_tiles - 1) / min_tiles;   // no range shorter than about min_tiles
   s.Peff = want < P ? want : P;
   s.fast = fast < 0 ? 0 : (fast < s.Peff ? fast : s.Peff);
-#ifndef EQUAL_SPLIT_BELOW
-#define EQUAL_SPLIT_BELOW 48
-#endif
   // short ranges are a matter of latency, which both workgroups of a compute unit see alike: equal shares
   if ((int64_t)s.T < (int64_t)EQUAL_SPLIT_BELOW * s.Peff) s.fast = 0;
   s.ctot = split_cum(s, s.Peff);

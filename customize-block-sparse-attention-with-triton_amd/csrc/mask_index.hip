@@ -133,8 +133,8 @@ __global__ __launch_bounds__(256) void fill_rows_kernel(const uint8_t* __restric
 // holds byte r * nb plus the set bits of that segment below it.  Lengths and the rows' positions in `groups`
 // follow from the starts after a second scan over the non-empty flags.
 // The same launch writes col_idx and groups: one workgroup writing 75 000 scattered entries would take 36-50 us, so
-// for masks of more than LISTS_FILL_MAX tiles the launch has 64 workgroups, each of which counts and scans the
-// whole mask for itself (75 KB from the L2) and fills a 64th of the entries.
+// for masks of more than LISTS_FILL_MAX tiles the launch has LISTS_FILL_WGS workgroups, each of which counts and scans the
+// whole mask for itself (75 KB from the L2) and fills its share of the entries.
 // ---------------------------------------------------------------------------------------
 constexpr int LISTS_ONE_MAX_ROWS = 1023, LISTS_ONE_MAX_SEG = 256;
 
@@ -163,6 +163,7 @@ __device__ __forceinline__ int block_inclusive_sum(int v, int* s_w, int* total) 
 // The kernel also writes col_idx and groups, every thread the entries of its own segment: with one workgroup for
 // masks of up to LISTS_FILL_MAX tiles, with several for larger ones (see below).
 constexpr int LISTS_FILL_MAX = 16384;
+constexpr int LISTS_FILL_WGS = 32;
 __global__ __launch_bounds__(1024) void count_scan_kernel(const uint8_t* __restrict__ block, int rows, int nb,
                                                           int seg, int32_t* __restrict__ row_ptr,
                                                           int32_t* __restrict__ gidx, int32_t* __restrict__ counts,
@@ -538,9 +539,6 @@ int launch_block_mask_to_lists(const uint8_t* block, int Bm, int Hm, int nb, int
   const dim3 grid((rows + 3) / 4);
   if (contiguous && rows <= LISTS_ONE_MAX_ROWS && total <= 1024 * LISTS_ONE_MAX_SEG) {
     const int seg = (((int)total + 1023) / 1024 + 15) / 16 * 16;
-#ifndef LISTS_FILL_WGS
-#define LISTS_FILL_WGS 32
-#endif
     // the whole call in one launch: one workgroup for small masks, LISTS_FILL_WGS for larger ones (each counts and
     // scans for itself and fills its share)
     hipLaunchKernelGGL(count_scan_kernel, dim3(total <= LISTS_FILL_MAX ? 1 : LISTS_FILL_WGS), dim3(1024), 0, st, block,
