@@ -726,6 +726,10 @@ void fwd_kernel(const FwdParams prm) {
         float wgt[NW][2];   // weight of wavefront p's partial for this lane's query of block qb
         float M[2], L[2];
         float keep[C::ROUNDS][C::QPW][4];   // this wavefront's share of the workgroup's part
+        // parts travel 16 bytes per lane and access at D = 64 (N = 17536, one head: dense 101.6 -> 101.0 us, keep 0.25
+        // 41.8 -> 41.1, keep 0.05 20.6 -> 20.0); at D = 128 that is faster for long ranges (keep 0.5 241 -> 233 us) and
+        // slower for short ones (keep 0.07 79 -> 82 us): 4 bytes there
+        constexpr bool WIDE_PARTS = D == 64;
         // A zero the compiler cannot see through (ctr[3] stays 0): the per-lane addresses into the
         // workspace do not change from row block to row block and would otherwise be computed
         // once, up front, and occupy registers throughout the tile loops.
@@ -737,6 +741,11 @@ void fwd_kernel(const FwdParams prm) {
           return prm.ws + (((int64_t)bh * prm.W + p) * 2 + (head ? 1 : 0)) * partial_floats(D) + zero;
         };
         float* slot = slot_of(wg, has_head);
+        // A part's holder looks at the arrival counter now: the value is only the first guess of the
+        // compare-and-swap below, and its round trip runs beside the merge instead of behind it.
+        unsigned long long* arrivals = prm.flags + (int64_t)bh * nb + r;
+        unsigned long long seen = 0;
+        if (!full && threadIdx.x == 0) seen = __hip_atomic_load(arrivals, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
         for (int rd = 0; rd < C::ROUNDS; ++rd) {
           {
@@ -785,8 +794,13 @@ void fwd_kernel(const FwdParams prm) {
               store_out4<BF16>(obase, qrow * prm.os[2] + 32 * db + 8 * i4 + 4 * g, prm.out_f32, x[0] * inv, x[1] * inv,
                                x[2] * inv, x[3] * inv);
             } else {
+              // (WIDE_PARTS: 16 bytes per lane and access, the part laid out [quad][lane][4])
+              if constexpr (WIDE_PARTS) {
+                coherent_store4(slot + idx0 * 64 + lane * 4, x[0], x[1], x[2], x[3]);
+              } else {
 #pragma unroll
-              for (int e = 0; e < 4; ++e) coherent_store(slot + (idx0 + e) * 64 + lane, x[e]);
+                for (int e = 0; e < 4; ++e) coherent_store(slot + (idx0 + e) * 64 + lane, x[e]);
+              }
             }
 #pragma unroll
             for (int e = 0; e < 4; ++e) keep[rd][tq][e] = x[e];
@@ -825,9 +839,8 @@ void fwd_kernel(const FwdParams prm) {
           // The counter holds (launch mark << 16 | parts counted); stale contents carry another mark.
           wait_vm<0>();
           __syncthreads();
-          unsigned long long* arrivals = prm.flags + (int64_t)bh * nb + r;
           if (threadIdx.x == 0) {
-            unsigned long long old = __hip_atomic_load(arrivals, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            unsigned long long old = seen;
             for (;;) {     // (ends: the counter only changes when another part is counted, at most nparts times)
               const unsigned long long want = (old >> 16) == prm.epoch ? old + 1 : ((prm.epoch << 16) | 1ull);
               if (__hip_atomic_compare_exchange_strong(arrivals, &old, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
@@ -869,14 +882,30 @@ void fwd_kernel(const FwdParams prm) {
                   mp[qb] = coherent_load(sp + 64 * D + qb * 32 + ln);
                   lp[qb] = coherent_load(sp + 64 * D + 64 + qb * 32 + ln);
                 }
+                if constexpr (WIDE_PARTS) {
+                  floatx4 ld[C::ROUNDS * C::QPW];
 #pragma unroll
-                for (int rd = 0; rd < C::ROUNDS; ++rd)
+                  for (int rd = 0; rd < C::ROUNDS; ++rd)
 #pragma unroll
-                  for (int tq = 0; tq < C::QPW; ++tq)
+                    for (int tq = 0; tq < C::QPW; ++tq)
+                      ld[rd * C::QPW + tq] = coherent_load4_issue(sp + (rd * C::R + 4 * (w * C::QPW + tq)) * 64 + lane * 4);
+                  coherent_loads_wait(ld);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                      dat[rd][tq][e] = coherent_load(sp + (rd * C::R + 4 * (w * C::QPW + tq) + e) * 64 + lane);
-                __builtin_amdgcn_sched_barrier(0);
+                  for (int rd = 0; rd < C::ROUNDS; ++rd)
+#pragma unroll
+                    for (int tq = 0; tq < C::QPW; ++tq)
+#pragma unroll
+                      for (int e = 0; e < 4; ++e) dat[rd][tq][e] = ld[rd * C::QPW + tq][e];
+                } else {
+#pragma unroll
+                  for (int rd = 0; rd < C::ROUNDS; ++rd)
+#pragma unroll
+                    for (int tq = 0; tq < C::QPW; ++tq)
+#pragma unroll
+                      for (int e = 0; e < 4; ++e)
+                        dat[rd][tq][e] = coherent_load(sp + (rd * C::R + 4 * (w * C::QPW + tq) + e) * 64 + lane);
+                  __builtin_amdgcn_sched_barrier(0);
+                }
               }
               float sc_own[2], sc_p[2];
 #pragma unroll
