@@ -728,7 +728,7 @@ void fwd_kernel(const FwdParams prm) {
         float keep[C::ROUNDS][C::QPW][4];   // this wavefront's share of the workgroup's part
         // parts travel 16 bytes per lane and access at D = 64 (N = 17536, one head: dense 101.6 -> 101.0 us, keep 0.25
         // 41.8 -> 41.1, keep 0.05 20.6 -> 20.0); at D = 128 that is faster for long ranges (keep 0.5 241 -> 233 us) and
-        // slower for short ones (keep 0.07 79 -> 82 us): 4 bytes there
+        // slower for short ones (keep 0.07 79 -> 82 us), and choosing by regime at run time gains nothing: 4 bytes there
         constexpr bool WIDE_PARTS = D == 64;
         // A zero the compiler cannot see through (ctr[3] stays 0): the per-lane addresses into the
         // workspace do not change from row block to row block and would otherwise be computed
