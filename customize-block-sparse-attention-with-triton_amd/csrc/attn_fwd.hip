@@ -883,13 +883,9 @@ void fwd_kernel(const FwdParams prm) {
                   lp[qb] = coherent_load(sp + 64 * D + 64 + qb * 32 + ln);
                 }
                 if constexpr (WIDE_PARTS) {
-                  floatx4 ld[C::ROUNDS * C::QPW];
-#pragma unroll
-                  for (int rd = 0; rd < C::ROUNDS; ++rd)
-#pragma unroll
-                    for (int tq = 0; tq < C::QPW; ++tq)
-                      ld[rd * C::QPW + tq] = coherent_load4_issue(sp + (rd * C::R + 4 * (w * C::QPW + tq)) * 64 + lane * 4);
-                  coherent_loads_wait(ld);
+                  static_assert(!WIDE_PARTS || (C::ROUNDS == 1 && C::QPW == 4), "four 16-byte loads per lane and part");
+                  floatx4 ld[4];
+                  coherent_load4x4(sp + 4 * (w * C::QPW) * 64 + lane * 4, ld[0], ld[1], ld[2], ld[3]);   // ([quad][lane][4]: a quad is 1 KB)
 #pragma unroll
                   for (int rd = 0; rd < C::ROUNDS; ++rd)
 #pragma unroll

@@ -214,22 +214,19 @@ __device__ __forceinline__ float coherent_load(const float* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 // The same accesses 16 bytes wide (p 16-byte aligned), written out, since an atomic type of that size does not
-// exist: `sc1` is what the compiler puts on the 4-byte ones above.  The compiler does not count these loads: the
-// values may be used after coherent_loads_wait on them, which waits for every vector memory access of the wavefront.
+// exist: `sc1` is what the compiler puts on the 4-byte ones above.
 __device__ __forceinline__ void coherent_store4(float* p, float a, float b, float c, float d) {
   const floatx4 v = {a, b, c, d};
   asm volatile("global_store_dwordx4 %0, %1, off sc1" :: "v"(p), "v"(v) : "memory");
 }
-__device__ __forceinline__ floatx4 coherent_load4_issue(const float* p) {
-  floatx4 v;
-  asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
-  return v;
-}
-template <int N> __device__ __forceinline__ void coherent_loads_wait(floatx4 (&x)[N]) {
-  static_assert(N % 4 == 0, "values are tied to the wait four at a time");
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#pragma unroll
-  for (int i = 0; i < N; i += 4) asm volatile("" : "+v"(x[i]), "+v"(x[i + 1]), "+v"(x[i + 2]), "+v"(x[i + 3]) :: "memory");
+// Four such loads, 1 KB apart, and the wait for them (and for every earlier vector memory access of the wavefront)
+// in one statement: the compiler does not count loads it did not issue, so the values must not leave the statement
+// before they have arrived.
+__device__ __forceinline__ void coherent_load4x4(const float* p, floatx4& a, floatx4& b, floatx4& c, floatx4& d) {
+  asm volatile("global_load_dwordx4 %0, %4, off sc1\n\tglobal_load_dwordx4 %1, %4, off offset:1024 sc1\n\t"
+               "global_load_dwordx4 %2, %4, off offset:2048 sc1\n\tglobal_load_dwordx4 %3, %4, off offset:3072 sc1\n\t"
+               "s_waitcnt vmcnt(0)"
+               : "=&v"(a), "=&v"(b), "=&v"(c), "=&v"(d) : "v"(p) : "memory");
 }
 
 // Swizzle for tiles that are read both ways (operand reads of 32 consecutive rows and
